@@ -31,7 +31,7 @@ extern "C" {
 
 /* Bumped whenever a signature or a semantic of this header changes; ssd_abi_version() returns the value the library was built
  * with, so a consumer compiled against another header can tell (tests/abi_consumer.c does). */
-#define SSD_HIP_ABI_VERSION 4
+#define SSD_HIP_ABI_VERSION 5
 
 #define SSD_OK 0
 #define SSD_ERR_SHAPE (-1)
@@ -485,6 +485,73 @@ int ssd_lightning_gate_norm(const void* o_rows, const void* proj_rows, long ld, 
  * the chosen + 1e-20) * scale. */
 int ssd_moe_route_softmax(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, int groups, int keep,
                           float scale, void* stream);
+
+/* Pre-norm layers over an fp32 residual stream (csrc/prenorm.hip).  ssd_embed_pos_res32: x (fp32 [T][W]) = table[ids[t]] +
+ * pos_table[positions[t]] (a learned position vector per position, unscaled; an id or position out of range gives a zero row) and,
+ * when norm_weight is given, norm_out = norm_weight * x / sqrt(mean(x^2) + eps) as element-type rows.
+ * ssd_prenorm_tail: x += y_rows (fp32 [T][W]) or, when y_rows is NULL, sum_j (weights ? weights[t*top+j] : 1) * ydn_rows[inv[t*top+j]];
+ * then (optional) next_out = next_weight * rms(x), the input rows of the next sublayer's first GEMM. */
+int ssd_embed_pos_res32(const int64_t* ids, const int64_t* positions, const void* table, const void* pos_table, void* x_out,
+                        const void* norm_weight, float eps, void* norm_out, int T, int W, long vocab, long max_pos, int f32,
+                        void* stream);
+int ssd_prenorm_tail(void* x, const void* y_rows, const void* ydn_rows, const int32_t* inv, const float* weights, int top, float eps,
+                     const void* next_weight, void* next_out, int T, int W, int f32, void* stream);
+/* out[t] = coef[0] rms(z) + coef[1] rms(z^2) + coef[2] rms(z^3) + coef[3] over fp32 rows [T][F] (powers element by element, rms(v) =
+ * v / sqrt(mean(v^2) + eps) per row), element-type rows out; coef: four fp32 numbers in device memory. */
+int ssd_polynorm_rows(const void* z_rows, const float* coef, float eps, void* out_rows, int T, int F, int f32, void* stream);
+/* Clamped swish-GLU over fp32 rows [rows][2F] = [zg | zu]: s = row_scale ? row_scale[perm ? perm[r] : r] : 1; g = min(s zg, limit),
+ * u = clamp(s zu, -limit, limit); out = g * sigmoid(alpha * g) * (u + 1), element-type rows [rows][F]. */
+int ssd_glu_clamp_rows(const void* ab_rows, const float* row_scale, const int32_t* perm, void* out_rows, int rows, int F, float limit,
+                       float alpha, int f32, void* stream);
+/* fp32 logit rows in place: z = scale * z, then (cap > 0) z = cap * tanh(z / cap). */
+int ssd_logits_cap_rows(void* logits, int rows, int V, long ld, float scale, float cap, void* stream);
+/* Router of the sigmoid kind: scores = sigmoid(logits[t][0..E)) (row stride ld), the `top` largest (lowest index wins a tie) -> idx,
+ * weights = those scores as they are. */
+int ssd_moe_route_sigmoid(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, void* stream);
+
+/* Sliding-window attention with unit-RMS q / k, capped scores, a per-head distance penalty and a softmax sink
+ * (csrc/attention_window.hip).  Store: qkv_rows fp32 [T][ld] = [q (H*D) | k (G*D) | v (G*Dv)]; q_out [T][H*D] = q / rms(q) per head;
+ * K cache [blocks][G][block_size][D] row slots[t] (-1: none) = k / rms(k); V cache [blocks][G][Dv][block_size] (transposed per page).
+ * Attention: out[t][h] (Dv wide) = sum_j p_j v_j over the keys j of the token's sequence with 0 <= positions[t] - j < window
+ * (window 0: all keys up to the token), s_j = cap * tanh(scale * <q, k_j> / cap) - slopes[h] * (positions[t] - j) (cap <= 0: no cap;
+ * slopes NULL: no penalty), p_j = exp(s_j) / (sum_j' exp(s_j') + exp(sinks[h])) (sinks NULL: no sink).  workspace (optional, fp32):
+ * with few rows the MFMA form cuts the window into key slices over the grid and merges them. */
+int ssd_winattn_store(const void* qkv_rows, long ld, float eps, const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int T,
+                      int H, int G, int D, int Dv, int block_size, int f32, void* stream);
+int ssd_winattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const float* slopes, const float* sinks,
+                      const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B,
+                      int T, int H, int G, int D, int Dv, int block_size, int window, float scale, float cap, void* out_rows, int f32,
+                      void* stream);
+
+/* Recurrent mixers over per-sequence state slots (csrc/recurrent.hip).  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows
+ * each; state_slots int32 [B]; a sequence whose first row has position 0 starts from zero whatever its slot holds.
+ * ssd_token_shift_mix: out[t][s] (W wide, s < S) = h + (h_prev - h) * mu[s] for element-type rows hn_rows [T][W]; h_prev = the row
+ * before in the batch, shift_state[slot] (fp32 [slots][W]) for a portion's first row, zero at position 0.
+ * ssd_wkv_scan: proj_rows fp32 [T][ld] holds r, k, v ([H][D] each) at r_off / k_off / v_off, decay_rows fp32 [T][ldw] the decay
+ * logits; per head w = exp(-exp(decay + w0)), o = (S + diag(u) k v^T)^T r, S = diag(w) S + k v^T over state fp32 [slots][H][D][D];
+ * out fp32 [T][H*D]; also shift_state[slot] = the sequence's last row of hn_rows.
+ * ssd_causal_conv_silu: out fp32 [T][C] = silu(conv_b[c] + sum_j conv_w[c][j] * in[t - (taps - 1 - j)][c]), in = proj_rows columns
+ * col_off .. col_off + C; inputs before a portion come from conv_state fp32 [slots][taps - 1][C] (last row = most recent).
+ * ssd_ssd_scan: per head (group h / (H / G)) dt = softplus(proj_rows[t][dt_off + h] + dt_bias[h]), S = exp(-exp(a_log[h]) dt) S +
+ * dt B x^T over state fp32 [slots][H][N][Dv], y = S^T C + skip[h] x; x / B / C = xbc_rows fp32 [T][ldx] at x_off ([H][Dv]), b_off,
+ * c_off ([G][N] each); out fp32 [T][H*Dv]; also saves the last taps - 1 rows of proj_rows columns conv_off .. conv_off + C into
+ * conv_state[slot].
+ * ssd_group_gate_norm: rows of N entries in `groups` equal parts, g = silu(gate_rows[t][c]) (fp32, row stride ldg): gate_first ?
+ * weight * rms_part(o * g) : weight * rms_part(o) * g, element-type rows. */
+int ssd_token_shift_mix(const void* hn_rows, const void* mu, const float* shift_state, const int64_t* positions, const int32_t* cu_q,
+                        int q_per_seq, const int32_t* state_slots, int B, void* out_rows, int T, int W, int S, int f32, void* stream);
+int ssd_wkv_scan(const void* proj_rows, long ld, int r_off, int k_off, int v_off, const void* decay_rows, long ldw, const float* w0,
+                 const float* u, const int64_t* positions, const int32_t* cu_q, int q_per_seq, const int32_t* state_slots, void* state,
+                 void* out_rows, const void* hn_rows, void* shift_state, int W, int B, int H, int D, int f32, void* stream);
+int ssd_causal_conv_silu(const void* proj_rows, long ld, int col_off, int C, const void* conv_w, const void* conv_b,
+                         const float* conv_state, const int64_t* positions, const int32_t* cu_q, int q_per_seq,
+                         const int32_t* state_slots, int B, void* out_rows, int T, int taps, int f32, void* stream);
+int ssd_ssd_scan(const void* xbc_rows, long ldx, int x_off, int b_off, int c_off, const void* proj_rows, long ld, int dt_off,
+                 const float* dt_bias, const float* a_log, const float* skip, const int64_t* positions, const int32_t* cu_q,
+                 int q_per_seq, const int32_t* state_slots, void* state, void* out_rows, int conv_off, int C, void* conv_state,
+                 int taps, int B, int H, int G, int N, int Dv, void* stream);
+int ssd_group_gate_norm(const void* o_rows, const void* gate_rows, long ldg, const void* weight, float eps, void* out_rows, int T,
+                        int N, int groups, int gate_first, int f32, void* stream);
 
 /* hipGraph capture for a host that is not PyTorch -- the reference captures its decode / verify / glue / tree steps with
  * torch.cuda.CUDAGraph (ssd/engine/helpers/cudagraph_helpers.py:20-120); every entry point above only enqueues on `stream`, so the calls

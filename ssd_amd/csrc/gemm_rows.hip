@@ -55,19 +55,21 @@ __device__ __forceinline__ void stage_tile(T* lds, const T* __restrict__ src, co
   }
 }
 
-// epilogue 0: fp32 rows; 1: relu(v)^2 as element-type rows; 2: element-type rows (3, 4: see glu_act)
+// epilogue 0: fp32 rows; 1: relu(v)^2 as element-type rows; 2: element-type rows; 5: tanh(v) as element-type rows (3, 4: see glu_act)
 template <typename T>
 __device__ __forceinline__ void store_out(void* y, long row, long ldy, long n, float v, int epi) {
   if (epi == 0) {
     reinterpret_cast<float*>(y)[row * ldy + n] = v;
   } else {
     if (epi == 1) { v = v > 0.f ? v : 0.f; v = v * v; }
+    if (epi == 5) v = tanhf(v);
     Elem<T>::st(reinterpret_cast<T*>(y) + row * ldy + n, v);
   }
 }
 
 // epilogues 3 / 4 (bf16 forms only): the weight rows come in (gate, up) pairs -- row 2i = gate_i, row 2i + 1 = up_i -- and the output is
 // act(gate) * up as element-type rows [M][N / 2], act = silu (3) or tanh-form gelu (4).  A lane's accumulators hold both halves of a pair.
+__host__ __device__ __forceinline__ bool epi_pairs(int epi) { return epi == 3 || epi == 4; }
 __device__ __forceinline__ float glu_act(float z, float u, int epi) {
   const float g = epi == 3 ? z / (1.0f + expf(-z)) : 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   return g * u;
@@ -119,7 +121,7 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
       __syncthreads();
     }
     const int m = row0 + wave * 16 + (lane & 15);
-    if (m < row_end && epi >= 3) {
+    if (m < row_end && epi_pairs(epi)) {
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
@@ -234,7 +236,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
       f32x4_t sum = red[lane];
 #pragma unroll
       for (int wv = 1; wv < NW; ++wv) sum += red[wv * 64 + lane];
-      if (mvalid && epi >= 3) {
+      if (mvalid && epi_pairs(epi)) {
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
           const int n = n0 + qd * 4 + e;
@@ -257,13 +259,13 @@ constexpr int SKINNY_MAX_ROWS = 16, SKINNY_MAX_GROUPED_ROWS = 64;
 int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, const int* offsets, int E, const int* row_idx,
            int idx_div, int f32, void* stream, int G = 1, long ldx = 0, long gsx = 0, long ldy = 0, long gsy = 0) {
   if (!x || !w || !y) return SSD_ERR_ARG;
-  if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 4) return SSD_ERR_SHAPE;
-  if (epi >= 3 && (f32 || (N & 1))) return SSD_ERR_SHAPE;        // the paired epilogues exist in the bf16 forms only
+  if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 5) return SSD_ERR_SHAPE;
+  if (epi_pairs(epi) && (f32 || (N & 1))) return SSD_ERR_SHAPE;        // the paired epilogues exist in the bf16 forms only
   if (offsets && E <= 0) return SSD_ERR_SHAPE;
   if (G < 1 || G > 65535 || (G > 1 && offsets)) return SSD_ERR_SHAPE;
   if (ldx == 0) ldx = K;
-  if (ldy == 0) ldy = epi >= 3 ? N / 2 : N;
-  if (ldx < K || ldy < (epi >= 3 ? N / 2 : N)) return SSD_ERR_SHAPE;
+  if (ldy == 0) ldy = epi_pairs(epi) ? N / 2 : N;
+  if (ldx < K || ldy < (epi_pairs(epi) ? N / 2 : N)) return SSD_ERR_SHAPE;
   const int esz0 = f32 ? 4 : 2;
   const bool x_vec = ((size_t)ldx * esz0) % 16 == 0 && ((size_t)gsx * esz0) % 16 == 0 && (uintptr_t)x % 16 == 0;
   if (!f32 && K % 8 == 0 && x_vec && (uintptr_t)w % 16 == 0 &&

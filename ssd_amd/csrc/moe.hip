@@ -4,6 +4,7 @@
 //   ssd_moe_route_softmax  the other common router: scores = softmax over ALL experts, experts in contiguous groups of which only the
 //                    best `keep` (by their largest score) stay eligible, the `top` largest eligible scores, divided by their sum
 //                    (+ 1e-20) and multiplied by a constant
+//   ssd_moe_route_sigmoid  scores = sigmoid of the logits, the `top` largest, weights = those scores unrenormalised
 //   ssd_moe_plan     counting sort of the T * top (token, slot) pairs by expert: offsets[E+1], perm (sorted row -> pair), inv (pair -> sorted row)
 //   ssd_moe_combine  out[t] = sum_j weight[t][j] * y[inv[t * top + j]] (+ shared[t]) in slot order, fp32
 // Between plan and combine the caller runs the experts as two grouped GEMMs over the sorted rows (up with the activation as epilogue,
@@ -97,6 +98,30 @@ moe_route_softmax_kernel(const float* __restrict__ zin, long ldz, int32_t* __res
   if (lane < top) wt[(size_t)t * top + lane] = myval / (sum + 1e-20f) * scale;
 }
 
+// Sigmoid routing: scores = sigmoid(logits), the `top` largest (lowest index wins a tie), weights = the chosen scores as they are
+// (no renormalisation).  One wave per token; logits row stride ldz.
+__global__ void __launch_bounds__(64)
+moe_route_sigmoid_kernel(const float* __restrict__ zin, long ldz, int32_t* __restrict__ idx, float* __restrict__ wt, int E, int top) {
+  extern __shared__ float z[];      // [E] scores
+  const int t = blockIdx.x, lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) z[e] = 1.0f / (1.0f + expf(-zin[(size_t)t * ldz + e]));
+  __syncthreads();
+  float myval = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY; int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) { const float v = z[e]; if (v > best) { best = v; bi = e; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if (lane == j % 64) { myval = best; idx[(size_t)t * top + j] = bi; }
+    if (lane == 0) z[bi] = -1.0f;      // scores are >= 0
+    __syncthreads();
+  }
+  if (lane < top) wt[(size_t)t * top + lane] = myval;
+}
+
 __global__ void __launch_bounds__(1024)
 moe_plan_kernel(const int32_t* __restrict__ idx, int n, int E, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
                 int32_t* __restrict__ inv) {
@@ -149,6 +174,13 @@ extern "C" int ssd_moe_route_softmax(const float* logits, long ld, int32_t* idx,
     return SSD_ERR_SHAPE;
   hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(T), dim3(64), (E + groups) * sizeof(float), (hipStream_t)stream, logits, ld, idx,
                      weights, E, top, groups, keep, scale);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_moe_route_sigmoid(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, void* stream) {
+  if (!logits || !idx || !weights) return SSD_ERR_ARG;
+  if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > E || top > MOE_MAX_TOP || ld < E) return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_sigmoid_kernel, dim3(T), dim3(64), E * sizeof(float), (hipStream_t)stream, logits, ld, idx, weights, E, top);
   return LAUNCH_OK();
 }
 

@@ -1,0 +1,345 @@
+// Recurrent mixers whose per-sequence memory is an fp32 matrix state per head plus a few rows of recent inputs, kept in the slot pool
+// that the block manager hands out (one slot per live sequence).  A forward reads a slot unless the rows it brings start at position 0,
+// walks its rows in order and writes the slot back, so a prompt may arrive in portions of any size; decoding is the one-row case.
+//
+//  token shift          ssd_token_shift_mix    mix_s = h + (h_prev - h) * mu_s for S interpolation vectors at once (h_prev: the previous
+//                                              token's row, from the batch, from the slot's saved row, or zero before position 0)
+//  time mixing ("wkv")  ssd_wkv_scan           per head, S [D][D]:  o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,  S_t = diag(w_t) S_(t-1) + k_t v_t^T,
+//                                              w_t = exp(-exp(ww_t + w0)) per key channel; also saves the slot's token-shift row
+//  short convolution    ssd_causal_conv_silu   out[c] = silu(b[c] + sum_j w[c][j] in_(t - (taps - 1 - j))[c]), inputs before the portion from
+//                                              the slot's saved rows, zero before position 0
+//  state space          ssd_ssd_scan           per head, S [N][Dv]:  S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t,
+//                                              dt_t = softplus(dt_raw + dt_bias) (no clamp); B / C shared by the heads of a group; also
+//                                              saves the slot's last taps - 1 convolution inputs
+//  output               ssd_group_gate_norm    RMS norm in `groups` equal parts of the row, a silu gate either BEFORE the norm (gate_first)
+//                                              or after it, times a weight, as GEMM-input rows
+// Everything that enters a recurrence is fp32: the projections' fp32 accumulators come in as fp32 rows, decays, step sizes, states and
+// sums stay fp32.  The arithmetic of a row does not depend on the portioning: per state element one multiply-add chain in token order,
+// the output a sum over the state rows in a fixed order.
+#include "common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, float v) { *p = (bf16_t)f2bf(v); }
+
+__device__ __forceinline__ float siluf_(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+__device__ __forceinline__ int seq_of_row(const int32_t* cu_q, int q_per_seq, int B, int t) {
+  if (!cu_q) return t / q_per_seq;
+  int lo = 0, hi = B;
+  while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (cu_q[mid] <= t) lo = mid; else hi = mid; }
+  return lo;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_mix_kernel(const T* __restrict__ hn, const T* __restrict__ mu, const float* __restrict__ shift_state,
+                       const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
+                       const int32_t* __restrict__ state_slots, int B, T* __restrict__ out, int W, int S) {
+  const int t = blockIdx.x;
+  const int b = seq_of_row(cu_q, q_per_seq, B, t);
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const bool from_batch = t > row0, zero = !from_batch && positions[t] == 0;
+  const float* st = shift_state + (size_t)state_slots[b] * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float h = ldf<T>(hn + (size_t)t * W + c);
+    const float prev = from_batch ? ldf<T>(hn + (size_t)(t - 1) * W + c) : (zero ? 0.f : st[c]);
+    for (int s = 0; s < S; ++s) stf<T>(out + ((size_t)t * S + s) * W + c, fmaf(prev - h, ldf<T>(mu + (size_t)s * W + c), h));
+  }
+}
+
+// One workgroup per (sequence, head).  Threads form NG groups of EP lanes (EP = power of two >= min(Dv, 256)): lane e of group g owns
+// the state elements (d, e) with d = g, g + NG, ...; the groups' partial outputs meet in LDS and are summed in group order.
+// MODE 0 (time mixing): the output reads the state BEFORE the update plus the bonus for the current token.
+// MODE 1 (state space): the output reads the state AFTER the update, plus skip * v.
+template <int MODE>
+__device__ __forceinline__ void scan_rows(float* S, const float* sq, const float* sk, const float* sd, const float* su, const float* sv,
+                                          float* po, int D, int Dv, int EP, float skip, float* out_row) {
+  const int tid = threadIdx.x, NG = 256 / EP, g = tid / EP, el = tid % EP;
+  for (int e = el; e < Dv; e += EP) {
+    const float ve = sv[e];
+    float o = 0.f;
+    for (int d = g; d < D; d += NG) {
+      const float s = S[d * Dv + e], kv = sk[d] * ve;
+      if (MODE == 0) {
+        o = fmaf(fmaf(su[d], kv, s), sq[d], o);
+        S[d * Dv + e] = fmaf(sd[d], s, kv);
+      } else {
+        const float n = fmaf(sd[d], s, kv);
+        S[d * Dv + e] = n;
+        o = fmaf(n, sq[d], o);
+      }
+    }
+    po[g * Dv + e] = o;
+  }
+  __syncthreads();
+  for (int e = tid; e < Dv; e += 256) {
+    float o = 0.f;
+    for (int gg = 0; gg < NG; ++gg) o += po[gg * Dv + e];
+    out_row[e] = MODE == 0 ? o : fmaf(skip, sv[e], o);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+wkv_scan_kernel(const float* __restrict__ proj, long ld, int r_off, int k_off, int v_off, const float* __restrict__ ww, long ldw,
+                const float* __restrict__ w0, const float* __restrict__ u, const int64_t* __restrict__ positions,
+                const int32_t* __restrict__ cu_q, int q_per_seq, const int32_t* __restrict__ state_slots, float* __restrict__ state,
+                float* __restrict__ out, const T* __restrict__ hn, float* __restrict__ shift_state, int W, int H, int D, int EP) {
+  extern __shared__ float lds[];
+  float* S = lds;                         // [D][D]
+  float* sq = S + (size_t)D * D;
+  float* sk = sq + D;
+  float* sd = sk + D;
+  float* su = sd + D;
+  float* sv = su + D;
+  float* po = sv + D;                     // [NG][D]
+  const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int row1 = cu_q ? cu_q[b + 1] : (b + 1) * q_per_seq;
+  if (row1 <= row0) return;
+  const int slot = state_slots[b];
+  float* sp = state + ((size_t)slot * H + h) * D * D;
+  const bool fresh = positions[row0] == 0;
+  for (int i = tid; i < D * D; i += 256) S[i] = fresh ? 0.f : sp[i];
+  for (int i = tid; i < D; i += 256) su[i] = u[h * D + i];
+  for (int r = row0; r < row1; ++r) {
+    const float* pr = proj + (size_t)r * ld + h * D;
+    __syncthreads();
+    for (int i = tid; i < D; i += 256) {
+      sq[i] = pr[r_off + i];
+      sk[i] = pr[k_off + i];
+      sv[i] = pr[v_off + i];
+      sd[i] = expf(-expf(ww[(size_t)r * ldw + h * D + i] + w0[h * D + i]));
+    }
+    __syncthreads();
+    scan_rows<0>(S, sq, sk, sd, su, sv, po, D, D, EP, 0.f, out + (size_t)r * H * D + h * D);
+  }
+  __syncthreads();
+  for (int i = tid; i < D * D; i += 256) sp[i] = S[i];
+  if (h == 0)          // the last row of the portion is the next portion's "previous token"
+    for (int c = tid; c < W; c += 256) shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+causal_conv_silu_kernel(const float* __restrict__ proj, long ld, int col_off, int C, const T* __restrict__ cw, const T* __restrict__ cb,
+                        const float* __restrict__ conv_state, const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
+                        int q_per_seq, const int32_t* __restrict__ state_slots, int B, float* __restrict__ out, int taps) {
+  const int t = blockIdx.x;
+  const int b = seq_of_row(cu_q, q_per_seq, B, t);
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const long p0 = positions[row0];
+  const float* st = conv_state + (size_t)state_slots[b] * (taps - 1) * C;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y) {
+    float acc = ldf<T>(cb + c);
+    for (int j = 0; j < taps; ++j) {
+      const int src = t - (taps - 1 - j);
+      float v;
+      if (src >= row0) {
+        v = proj[(size_t)src * ld + col_off + c];
+      } else {
+        const int k = row0 - src;                          // k tokens before the portion's first row
+        v = p0 - k >= 0 ? st[(size_t)(taps - 1 - k) * C + c] : 0.f;
+      }
+      acc = fmaf(ldf<T>(cw + (size_t)c * taps + j), v, acc);
+    }
+    out[(size_t)t * C + c] = siluf_(acc);
+  }
+}
+
+constexpr int CONV_MAX_TAPS = 16;
+
+__global__ void __launch_bounds__(256)
+ssd_scan_kernel(const float* __restrict__ xbc, long ldx, int x_off, int b_off, int c_off, const float* __restrict__ proj, long ld,
+                int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ dskip,
+                const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
+                const int32_t* __restrict__ state_slots, float* __restrict__ state, float* __restrict__ out, int conv_off, int C,
+                float* __restrict__ conv_state, int taps, int H, int G, int N, int Dv, int EP) {
+  extern __shared__ float lds[];
+  float* S = lds;                         // [N][Dv]
+  float* sq = S + (size_t)N * Dv;
+  float* sk = sq + N;
+  float* sd = sk + N;
+  float* sv = sd + N;                     // [Dv]
+  float* po = sv + Dv;                    // [NG][Dv]
+  const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int grp = h / (H / G);
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int row1 = cu_q ? cu_q[b + 1] : (b + 1) * q_per_seq;
+  if (row1 <= row0) return;
+  const int slot = state_slots[b];
+  float* sp = state + ((size_t)slot * H + h) * N * Dv;
+  const long p0 = positions[row0];
+  const bool fresh = p0 == 0;
+  for (int i = tid; i < N * Dv; i += 256) S[i] = fresh ? 0.f : sp[i];
+  const float a = -expf(a_log[h]), dtb = dt_bias[h], skip = dskip[h];
+  for (int r = row0; r < row1; ++r) {
+    const float* xr = xbc + (size_t)r * ldx;
+    const float dt = softplusf_(proj[(size_t)r * ld + dt_off + h] + dtb);
+    const float dA = expf(a * dt);
+    __syncthreads();
+    for (int i = tid; i < N; i += 256) {
+      sq[i] = xr[c_off + grp * N + i];
+      sk[i] = dt * xr[b_off + grp * N + i];
+      sd[i] = dA;
+    }
+    for (int i = tid; i < Dv; i += 256) sv[i] = xr[x_off + h * Dv + i];
+    __syncthreads();
+    scan_rows<1>(S, sq, sk, sd, nullptr, sv, po, N, Dv, EP, skip, out + (size_t)r * H * Dv + h * Dv);
+  }
+  __syncthreads();
+  for (int i = tid; i < N * Dv; i += 256) sp[i] = S[i];
+  if (h == 0 && taps > 1) {
+    // the slot's last taps - 1 convolution inputs: saved row i holds the input of position p0 + n - (taps - 1) + i
+    const int n = row1 - row0, K1 = taps - 1;
+    float* st = conv_state + (size_t)slot * K1 * C;
+    for (int c = tid; c < C; c += 256) {
+      float keep[CONV_MAX_TAPS];
+#pragma unroll
+      for (int i = 0; i < CONV_MAX_TAPS; ++i) {
+        keep[i] = 0.f;
+        if (i < K1) {
+          const long rel = (long)n - K1 + i;                // position relative to the portion's first row
+          if (rel >= 0) keep[i] = proj[(size_t)(row0 + rel) * ld + conv_off + c];
+          else if (p0 + rel >= 0) keep[i] = st[(size_t)(i + n) * C + c];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < CONV_MAX_TAPS; ++i)
+        if (i < K1) st[(size_t)i * C + c] = keep[i];
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_gate_norm_kernel(const float* __restrict__ o, const float* __restrict__ gate, long ldg, const T* __restrict__ w, float eps,
+                       T* __restrict__ out, int N, int groups, int gate_first) {
+  const size_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, per = N / groups;
+  const float* orow = o + t * N;
+  const float* grow = gate + t * ldg;
+  for (int g = blockIdx.y * 4 + wave; g < groups; g += 4 * gridDim.y) {
+    float ss = 0.f;
+    for (int c = g * per + lane; c < (g + 1) * per; c += 64) {
+      const float v = gate_first ? orow[c] * siluf_(grow[c]) : orow[c];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)per + eps);
+    for (int c = g * per + lane; c < (g + 1) * per; c += 64) {
+      const float gs = siluf_(grow[c]);
+      const float v = gate_first ? orow[c] * gs * r * ldf<T>(w + c) : orow[c] * r * ldf<T>(w + c) * gs;
+      stf<T>(out + t * N + c, v);
+    }
+  }
+}
+
+int pick_ep(int Dv) {
+  int EP = 1;
+  while (EP < Dv && EP < 256) EP <<= 1;
+  return EP;
+}
+
+}  // namespace
+
+#define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
+
+extern "C" int ssd_token_shift_mix(const void* hn_rows, const void* mu, const float* shift_state, const int64_t* positions,
+                                   const int32_t* cu_q, int q_per_seq, const int32_t* state_slots, int B, void* out_rows, int T, int W,
+                                   int S, int f32, void* stream) {
+  if (!hn_rows || !mu || !shift_state || !positions || !state_slots || !out_rows) return SSD_ERR_ARG;
+  if (T <= 0 || W <= 0 || S <= 0 || B <= 0 || (!cu_q && q_per_seq <= 0)) return SSD_ERR_SHAPE;
+  if (f32)
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)hn_rows, (const float*)mu,
+                       shift_state, positions, cu_q, q_per_seq, state_slots, B, (float*)out_rows, W, S);
+  else
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)hn_rows,
+                       (const bf16_t*)mu, shift_state, positions, cu_q, q_per_seq, state_slots, B, (bf16_t*)out_rows, W, S);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_wkv_scan(const void* proj_rows, long ld, int r_off, int k_off, int v_off, const void* decay_rows, long ldw,
+                            const float* w0, const float* u, const int64_t* positions, const int32_t* cu_q, int q_per_seq,
+                            const int32_t* state_slots, void* state, void* out_rows, const void* hn_rows, void* shift_state, int W,
+                            int B, int H, int D, int f32, void* stream) {
+  if (!proj_rows || !decay_rows || !w0 || !u || !positions || !state_slots || !state || !out_rows || !hn_rows || !shift_state)
+    return SSD_ERR_ARG;
+  if (B <= 0 || H <= 0 || D <= 0 || W <= 0 || (!cu_q && q_per_seq <= 0) || H > 65535) return SSD_ERR_SHAPE;
+  const int EP = pick_ep(D);
+  const size_t bytes = ((size_t)D * D + 6 * (size_t)D + (size_t)(256 / EP) * D) * sizeof(float);
+  if (bytes > 160 * 1024) return SSD_ERR_SHAPE;
+  const void* fn = f32 ? (const void*)wkv_scan_kernel<float> : (const void*)wkv_scan_kernel<bf16_t>;
+  if (bytes > 64 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+    return SSD_ERR_LAUNCH;
+  if (f32)
+    hipLaunchKernelGGL(wkv_scan_kernel<float>, dim3(B, H), dim3(256), bytes, (hipStream_t)stream, (const float*)proj_rows, ld, r_off,
+                       k_off, v_off, (const float*)decay_rows, ldw, w0, u, positions, cu_q, q_per_seq, state_slots, (float*)state,
+                       (float*)out_rows, (const float*)hn_rows, (float*)shift_state, W, H, D, EP);
+  else
+    hipLaunchKernelGGL(wkv_scan_kernel<bf16_t>, dim3(B, H), dim3(256), bytes, (hipStream_t)stream, (const float*)proj_rows, ld, r_off,
+                       k_off, v_off, (const float*)decay_rows, ldw, w0, u, positions, cu_q, q_per_seq, state_slots, (float*)state,
+                       (float*)out_rows, (const bf16_t*)hn_rows, (float*)shift_state, W, H, D, EP);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_causal_conv_silu(const void* proj_rows, long ld, int col_off, int C, const void* conv_w, const void* conv_b,
+                                    const float* conv_state, const int64_t* positions, const int32_t* cu_q, int q_per_seq,
+                                    const int32_t* state_slots, int B, void* out_rows, int T, int taps, int f32, void* stream) {
+  if (!proj_rows || !conv_w || !conv_b || !conv_state || !positions || !state_slots || !out_rows) return SSD_ERR_ARG;
+  if (T <= 0 || C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || B <= 0 || (!cu_q && q_per_seq <= 0) || ld < col_off + C) return SSD_ERR_SHAPE;
+  const int cb = (C + 255) / 256;
+  const dim3 grid(T, cb < 64 ? cb : 64);
+  if (f32)
+    hipLaunchKernelGGL(causal_conv_silu_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, col_off, C,
+                       (const float*)conv_w, (const float*)conv_b, conv_state, positions, cu_q, q_per_seq, state_slots, B,
+                       (float*)out_rows, taps);
+  else
+    hipLaunchKernelGGL(causal_conv_silu_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, col_off, C,
+                       (const bf16_t*)conv_w, (const bf16_t*)conv_b, conv_state, positions, cu_q, q_per_seq, state_slots, B,
+                       (float*)out_rows, taps);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_ssd_scan(const void* xbc_rows, long ldx, int x_off, int b_off, int c_off, const void* proj_rows, long ld, int dt_off,
+                            const float* dt_bias, const float* a_log, const float* skip, const int64_t* positions, const int32_t* cu_q,
+                            int q_per_seq, const int32_t* state_slots, void* state, void* out_rows, int conv_off, int C,
+                            void* conv_state, int taps, int B, int H, int G, int N, int Dv, void* stream) {
+  if (!xbc_rows || !proj_rows || !dt_bias || !a_log || !skip || !positions || !state_slots || !state || !out_rows || !conv_state)
+    return SSD_ERR_ARG;
+  if (B <= 0 || H <= 0 || G <= 0 || H % G || N <= 0 || Dv <= 0 || taps < 1 || taps > CONV_MAX_TAPS || C <= 0 ||
+      (!cu_q && q_per_seq <= 0) || H > 65535)
+    return SSD_ERR_SHAPE;
+  const int EP = pick_ep(Dv);
+  const size_t bytes = ((size_t)N * Dv + 3 * (size_t)N + Dv + (size_t)(256 / EP) * Dv) * sizeof(float);
+  if (bytes > 160 * 1024) return SSD_ERR_SHAPE;
+  if (bytes > 64 * 1024 &&
+      hipFuncSetAttribute((const void*)ssd_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+    return SSD_ERR_LAUNCH;
+  hipLaunchKernelGGL(ssd_scan_kernel, dim3(B, H), dim3(256), bytes, (hipStream_t)stream, (const float*)xbc_rows, ldx, x_off, b_off, c_off,
+                     (const float*)proj_rows, ld, dt_off, dt_bias, a_log, skip, positions, cu_q, q_per_seq, state_slots, (float*)state,
+                     (float*)out_rows, conv_off, C, (float*)conv_state, taps, H, G, N, Dv, EP);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_group_gate_norm(const void* o_rows, const void* gate_rows, long ldg, const void* weight, float eps, void* out_rows,
+                                   int T, int N, int groups, int gate_first, int f32, void* stream) {
+  if (!o_rows || !gate_rows || !weight || !out_rows) return SSD_ERR_ARG;
+  if (T <= 0 || N <= 0 || groups <= 0 || N % groups || ldg < N) return SSD_ERR_SHAPE;
+  const int gb = (groups + 3) / 4;
+  const dim3 grid(T, T >= 256 ? 1 : (gb < 16 ? gb : 16));
+  if (f32)
+    hipLaunchKernelGGL(group_gate_norm_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)o_rows,
+                       (const float*)gate_rows, ldg, (const float*)weight, eps, (float*)out_rows, N, groups, gate_first);
+  else
+    hipLaunchKernelGGL(group_gate_norm_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)o_rows,
+                       (const float*)gate_rows, ldg, (const bf16_t*)weight, eps, (bf16_t*)out_rows, N, groups, gate_first);
+  return LAUNCH_OK();
+}

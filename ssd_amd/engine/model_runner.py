@@ -37,6 +37,9 @@ def model_class(family: str):
     if family == "zerusun":
         from ssd_amd.zerusun import HipZerusun
         return HipZerusun
+    if family == "fomunex":
+        from ssd_amd.fomunex import HipFomunex
+        return HipFomunex
     return HipDecoder
 
 

@@ -16,7 +16,7 @@ _LIB = None
 
 c_void_p, c_int, c_long, c_float, c_int64 = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_int64
 
-ABI_VERSION = 4       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
+ABI_VERSION = 5       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
 
 # name -> argtypes, exactly include/ssd_hip.h (+ include/ssd_hip_tune.h)
 SIGNATURES = {
@@ -142,6 +142,26 @@ SIGNATURES = {
                            c_int, c_int, c_int, c_int, c_void_p],
     "ssd_lightning_gate_norm": [c_void_p, c_void_p, c_long, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_moe_route_softmax": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ssd_embed_pos_res32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_long, c_long,
+                            c_int, c_void_p],
+    "ssd_prenorm_tail": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_polynorm_rows": [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_glu_clamp_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    "ssd_logits_cap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_float, c_void_p],
+    "ssd_moe_route_sigmoid": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_winattn_store": [c_void_p, c_long, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                          c_int, c_void_p],
+    "ssd_winattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p],
+    "ssd_token_shift_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                            c_int, c_void_p],
+    "ssd_wkv_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                     c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_causal_conv_silu": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                             c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_ssd_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                     c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_group_gate_norm": [c_void_p, c_void_p, c_long, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ssd_draft_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_void_p, c_int, c_void_p],
 }
@@ -157,6 +177,7 @@ _COMMON_ROWS = ["misc.hip", "gemm_rows.hip", "res32.hip", "moe.hip", "sample.hip
 FAMILY_SOURCES = {
     "fatulix": _COMMON_ROWS + ["attention_diff.hip"],
     "zerusun": _COMMON_ROWS + ["dyt.hip", "attention_latent.hip", "lightning.hip"],
+    "fomunex": _COMMON_ROWS + ["prenorm.hip", "attention_window.hip", "recurrent.hip"],
 }
 
 

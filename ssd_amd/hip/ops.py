@@ -519,3 +519,84 @@ def lightning_gate_norm(o_rows, proj, ld: int, g_off: int, weight, eps: float, o
 def moe_route_softmax(logits, ld: int, idx, weights, T: int, E: int, top: int, groups: int, keep: int, scale: float):
     _check(load_library().ssd_moe_route_softmax(_p(logits), ld, _p(idx), _p(weights), T, E, top, groups, keep, scale, _stream()),
            "ssd_moe_route_softmax")
+
+
+# ---- pre-norm layers over an fp32 residual, windowed attention with a sink, recurrent mixers (time mixing, state space) ----
+
+GR_TANH = 5
+
+
+def embed_pos_res32(ids, positions, table, pos_table, x_out, T: int, W: int, f32: bool, norm_weight=None, eps: float = 0.0, norm_out=None):
+    _check(load_library().ssd_embed_pos_res32(_p(ids), _p(positions), _p(table), _p(pos_table), _p(x_out), _p(norm_weight), eps,
+                                              _p(norm_out), T, W, table.shape[0], pos_table.shape[0], int(f32), _stream()),
+           "ssd_embed_pos_res32")
+
+
+def prenorm_tail(x, eps: float, T: int, W: int, f32: bool, *, y=None, ydn=None, inv=None, weights=None, top: int = 0, next_weight=None,
+                 next_out=None):
+    """x += y (fp32 rows) or the sum of a token's expert rows ydn[inv[t * top + j]] (times weights when given); next_out = next_weight * rms(x)."""
+    _check(load_library().ssd_prenorm_tail(_p(x), _p(y), _p(ydn), _p(inv), _p(weights), top, eps, _p(next_weight), _p(next_out), T, W,
+                                           int(f32), _stream()), "ssd_prenorm_tail")
+
+
+def polynorm_rows(z, coef, eps: float, out_rows, T: int, F: int, f32: bool):
+    _check(load_library().ssd_polynorm_rows(_p(z), _p(coef), eps, _p(out_rows), T, F, int(f32), _stream()), "ssd_polynorm_rows")
+
+
+def glu_clamp_rows(ab, out_rows, rows: int, F: int, limit: float, alpha: float, f32: bool, row_scale=None, perm=None):
+    _check(load_library().ssd_glu_clamp_rows(_p(ab), _p(row_scale), _p(perm), _p(out_rows), rows, F, limit, alpha, int(f32), _stream()),
+           "ssd_glu_clamp_rows")
+
+
+def logits_cap_rows(logits, rows: int, V: int, ld: int, scale: float, cap: float):
+    _check(load_library().ssd_logits_cap_rows(_p(logits), rows, V, ld, scale, cap, _stream()), "ssd_logits_cap_rows")
+
+
+def moe_route_sigmoid(logits, ld: int, idx, weights, T: int, E: int, top: int):
+    _check(load_library().ssd_moe_route_sigmoid(_p(logits), ld, _p(idx), _p(weights), T, E, top, _stream()), "ssd_moe_route_sigmoid")
+
+
+def winattn_store(qkv, ld: int, eps: float, slots, q_out, k_cache, v_cache, T: int, H: int, G: int, D: int, Dv: int, block_size: int,
+                  f32: bool):
+    _check(load_library().ssd_winattn_store(_p(qkv), ld, eps, _p(slots), _p(q_out), _p(k_cache), _p(v_cache), T, H, G, D, Dv, block_size,
+                                            int(f32), _stream()), "ssd_winattn_store")
+
+
+def winattn_paged(q, k_cache, v_cache, slopes, sinks, block_tables, max_blocks: int, positions, B: int, T: int, H: int, G: int, D: int,
+                  Dv: int, block_size: int, window: int, scale: float, cap: float, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_winattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(slopes), _p(sinks), _p(block_tables), max_blocks,
+                                            _p(positions), _p(cu_q), q_per_seq, B, T, H, G, D, Dv, block_size, window, scale, cap,
+                                            _p(out_rows), int(f32), _stream()), "ssd_winattn_paged")
+
+
+def token_shift_mix(hn, mu, shift_state, positions, state_slots, B: int, out_rows, T: int, W: int, S: int, f32: bool, cu_q=None,
+                    q_per_seq: int = 0):
+    _check(load_library().ssd_token_shift_mix(_p(hn), _p(mu), _p(shift_state), _p(positions), _p(cu_q), q_per_seq, _p(state_slots), B,
+                                              _p(out_rows), T, W, S, int(f32), _stream()), "ssd_token_shift_mix")
+
+
+def wkv_scan(proj, ld: int, r_off: int, k_off: int, v_off: int, decay_rows, ldw: int, w0, u, positions, state_slots, state, out_rows,
+             hn, shift_state, W: int, B: int, H: int, D: int, f32: bool, cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_wkv_scan(_p(proj), ld, r_off, k_off, v_off, _p(decay_rows), ldw, _p(w0), _p(u), _p(positions), _p(cu_q),
+                                       q_per_seq, _p(state_slots), _p(state), _p(out_rows), _p(hn), _p(shift_state), W, B, H, D,
+                                       int(f32), _stream()), "ssd_wkv_scan")
+
+
+def causal_conv_silu(proj, ld: int, col_off: int, C: int, conv_w, conv_b, conv_state, positions, state_slots, B: int, out_rows, T: int,
+                     taps: int, f32: bool, cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_causal_conv_silu(_p(proj), ld, col_off, C, _p(conv_w), _p(conv_b), _p(conv_state), _p(positions), _p(cu_q),
+                                               q_per_seq, _p(state_slots), B, _p(out_rows), T, taps, int(f32), _stream()),
+           "ssd_causal_conv_silu")
+
+
+def ssd_scan(xbc, ldx: int, x_off: int, b_off: int, c_off: int, proj, ld: int, dt_off: int, dt_bias, a_log, skip, positions, state_slots,
+             state, out_rows, conv_off: int, C: int, conv_state, taps: int, B: int, H: int, G: int, N: int, Dv: int, cu_q=None,
+             q_per_seq: int = 0):
+    _check(load_library().ssd_ssd_scan(_p(xbc), ldx, x_off, b_off, c_off, _p(proj), ld, dt_off, _p(dt_bias), _p(a_log), _p(skip),
+                                       _p(positions), _p(cu_q), q_per_seq, _p(state_slots), _p(state), _p(out_rows), conv_off, C,
+                                       _p(conv_state), taps, B, H, G, N, Dv, _stream()), "ssd_ssd_scan")
+
+
+def group_gate_norm(o_rows, gate_rows, ldg: int, weight, eps: float, out_rows, T: int, N: int, groups: int, gate_first: bool, f32: bool):
+    _check(load_library().ssd_group_gate_norm(_p(o_rows), _p(gate_rows), ldg, _p(weight), eps, _p(out_rows), T, N, groups,
+                                              int(gate_first), int(f32), _stream()), "ssd_group_gate_norm")

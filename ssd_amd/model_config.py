@@ -351,8 +351,176 @@ class ZerusunConfig:
         return out
 
 
+# --------------------------------------------------------------------------------------------------
+# Fomunex: pre-norm layers (one-number RMS norms) over an fp32 residual with a learned position vector; mixers are windowed attention
+# with a sink, RWKV-style time mixing, or a Mamba-2 state space; feed-forwards are PolyNorm dense or sigmoid-routed clamped GLUs
+# --------------------------------------------------------------------------------------------------
+@dataclass
+class WindowAttention:
+    """Grouped-query attention without rotation: q and k divided by their root mean square per head, scores scale * <q, k> capped by
+    softcap * tanh(. / softcap) (0: no cap), minus slope_h * distance with slope_h = 2^(-8 (h + 1) / heads), a sliding window (a token
+    sees itself and the window - 1 tokens before it; 0: every earlier token) and a learned per-head sink in the softmax denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0
+    window: int = 0
+    kind: str = "attention"
+
+    def slopes(self) -> list[float]:
+        return [2.0 ** (-8.0 * (h + 1) / self.heads) for h in range(self.heads)]
+
+
+@dataclass
+class WkvMixer:
+    """RWKV-style time mixing: r, k, v, gate and the decay each read their own interpolation between the token's row and the previous
+    token's; per head a [dim][dim] fp32 state with a per-channel data-dependent decay exp(-exp(W_w2 tanh(W_w1 mix) + w0)) and a bonus
+    for the current token; per-head unit-RMS output, silu gate.  decay_rank: the inner size of the decay's two matrices (a tensor's
+    shape, not a config.json key: 0 until a checkpoint's header or the caller gives it)."""
+    heads: int
+    dim: int
+    decay_rank: int = 0
+    kind: str = "wkv"
+
+
+@dataclass
+class Mamba2Mixer:
+    """Mamba-2 state space: inner = heads * vdim channels, a [state][vdim] fp32 state per head with one decay per head and token,
+    B / C shared by the heads of one of `groups` groups, a causal convolution of `conv` taps over [x | B | C], the silu gate applied
+    BEFORE an RMS norm in `norm_groups` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+    kind: str = "mamba2"
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass
+class PolyNormMLP:
+    """Dense feed-forward W_down act(W_up h) with act(z) = a rms(z) + b rms(z^2) + c rms(z^3) + e over a token's ff values."""
+    ff: int
+    kind: str = "dense"
+
+
+@dataclass
+class SigmoidRoutedMLP:
+    """Mixture of experts with a sigmoid router: the `top` largest scores, unrenormalised, each multiplying its expert's INPUT; experts
+    g = min(W_gate h, limit), u = clamp(W_up h, +-limit), W_down (g sigmoid(1.702 g) (u + 1))."""
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    kind: str = "moe"
+
+
+@dataclass
+class FomunexLayer:
+    mixer: object               # WindowAttention | WkvMixer | Mamba2Mixer
+    mlp: object                 # PolyNormMLP | SigmoidRoutedMLP | None
+    weights_of: int             # the layer whose tensors this layer uses (itself unless config.json says otherwise); cache / state are its own
+
+
+@dataclass
+class FomunexConfig:
+    """config.json keys: architecture, vocab, width, max_positions, norm.eps, logit_scale, logit_softcap, layers[{type, mixer{...},
+    mlp{kind, ...} | null, weights_of?}]."""
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float
+    layers: list = field(default_factory=list)
+    max_position_embeddings: int = 2048
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
+    family: str = "fomunex"
+    tie_word_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def recurrent(self) -> bool:
+        """True when some layer keeps a per-sequence state that is not a function of cached pages."""
+        return any(l.mixer.kind in ("wkv", "mamba2") for l in self.layers)
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+    def complete_from_checkpoint(self, model_dir: str) -> None:
+        """Sizes that only a tensor's shape gives (the decay rank of time-mixing layers): read from the safetensors headers."""
+        need = [i for i, l in enumerate(self.layers) if l.mixer.kind == "wkv" and not l.mixer.decay_rank]
+        if not need:
+            return
+        import glob
+        import struct
+        shapes = {}
+        for f in sorted(glob.glob(os.path.join(model_dir, "*.safetensors"))):
+            with open(f, "rb") as fh:
+                n = struct.unpack("<Q", fh.read(8))[0]
+                shapes.update({k: v.get("shape") for k, v in json.loads(fh.read(n)).items() if k != "__metadata__"})
+        for i in need:
+            name = f"l{self.layers[i].weights_of}.mix.w1"
+            if name not in shapes:
+                raise ValueError(f"Fomunex: {name} not found under {model_dir}")
+            self.layers[i].mixer.decay_rank = int(shapes[name][0])
+
+    @staticmethod
+    def from_json(cfg: dict) -> "FomunexConfig":
+        layers = []
+        for i, lc in enumerate(cfg["layers"]):
+            m, kind = lc["mixer"], lc["type"]
+            if kind == "attention":
+                mask = m.get("mask") or {}
+                mixer = WindowAttention(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]),
+                                        float(m.get("softcap") or 0.0), int(mask.get("size") or 0))
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError("Fomunex: heads must be a multiple of kv_heads")
+            elif kind == "wkv":
+                mixer = WkvMixer(int(m["heads"]), int(m["dim"]), int(m.get("decay_rank") or 0))
+            elif kind == "mamba2":
+                mixer = Mamba2Mixer(int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups", 1)), int(m["conv"]),
+                                    int(m.get("norm_groups", 1)))
+                if mixer.heads % mixer.groups or mixer.inner % mixer.norm_groups or mixer.conv < 1:
+                    raise ValueError("Fomunex: state-space groups do not fit the heads")
+            else:
+                raise ValueError(f"Fomunex: unknown layer type {kind!r}")
+            ml = lc.get("mlp")
+            mlp = None
+            if ml is not None:
+                if ml["kind"] == "dense":
+                    mlp = PolyNormMLP(int(ml["ff"]))
+                elif ml["kind"] == "moe":
+                    mlp = SigmoidRoutedMLP(int(ml["router"]["experts"]), int(ml["router"]["top"]), int(ml["expert"]["ff"]),
+                                           float(ml["expert"]["limit"]))
+                    if not 1 <= mlp.top <= mlp.experts:
+                        raise ValueError("Fomunex: top does not fit the experts")
+                else:
+                    raise ValueError(f"Fomunex: unknown feed-forward kind {ml['kind']!r}")
+            src = int(lc.get("weights_of", i))
+            if not 0 <= src < len(cfg["layers"]) or cfg["layers"][src].get("weights_of", src) != src or cfg["layers"][src]["type"] != kind:
+                raise ValueError(f"Fomunex: layer {i} cannot use the weights of layer {src}")
+            layers.append(FomunexLayer(mixer, mlp, src))
+        for l in layers:        # a layer that borrows weights has its source's sizes, also the one a tensor's shape gives
+            if l.mixer.kind == "wkv" and not l.mixer.decay_rank:
+                l.mixer.decay_rank = layers[l.weights_of].mixer.decay_rank
+        return FomunexConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, int(cfg["max_positions"]),
+                             float(cfg.get("logit_scale", 1.0)), float(cfg.get("logit_softcap") or 0.0))
+
+
 # config.json "architecture" values that are read by this package's own readers (everything else goes through transformers' AutoConfig)
-ARCHITECTURES = {"Fatulix": FatulixConfig.from_json, "Zerusun": ZerusunConfig.from_json}
+ARCHITECTURES = {"Fatulix": FatulixConfig.from_json, "Zerusun": ZerusunConfig.from_json, "Fomunex": FomunexConfig.from_json}
 
 
 def read_native_config(model_dir: str):
@@ -363,4 +531,9 @@ def read_native_config(model_dir: str):
     with open(path) as f:
         cfg = json.load(f)
     reader = ARCHITECTURES.get(cfg.get("architecture")) if isinstance(cfg, dict) else None
-    return reader(cfg) if reader else None
+    if not reader:
+        return None
+    out = reader(cfg)
+    if hasattr(out, "complete_from_checkpoint"):      # sizes that only a tensor's shape gives
+        out.complete_from_checkpoint(model_dir)
+    return out

@@ -103,6 +103,41 @@ def zerusun_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
     return out + norm("final.norm")
 
 
+def fomunex_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
+    """Tensor names and shapes of a Fomunex checkpoint (model_config.FomunexConfig).  Norm weights are single numbers (shape ()); a
+    layer that uses another layer's weights has no tensors of its own."""
+    W = cfg.hidden_size
+    out = [("embed", (cfg.vocab_size, W)), ("pos", (cfg.max_position_embeddings, W))]
+    for i, lc in enumerate(cfg.layers):
+        if lc.weights_of != i:
+            continue
+        p, m, ml = f"l{i}.", lc.mixer, lc.mlp
+        out += [(p + "norm1", ())] + ([(p + "norm2", ())] if ml is not None else [])
+        if m.kind == "attention":
+            out += [(p + "mix.q", (m.heads * m.dim, W)), (p + "mix.k", (m.kv_heads * m.dim, W)), (p + "mix.v", (m.kv_heads * m.vdim, W)),
+                    (p + "mix.sink", (m.heads,)), (p + "mix.o", (W, m.heads * m.vdim))]
+        elif m.kind == "wkv":
+            n = m.heads * m.dim
+            assert m.decay_rank > 0, "a time-mixing layer needs its decay rank (a checkpoint's tensor shape or WkvMixer.decay_rank)"
+            out += [(p + f"mix.mu.{s}", (W,)) for s in "rkvgw"]
+            out += [(p + f"mix.{s}", (n, W)) for s in "rkvg"]
+            out += [(p + "mix.w1", (m.decay_rank, W)), (p + "mix.w2", (n, m.decay_rank)), (p + "mix.w0", (n,)), (p + "mix.u", (m.heads, m.dim)),
+                    (p + "mix.norm", (n,)), (p + "mix.o", (W, n))]
+        else:
+            out += [(p + "mix.in", (2 * m.inner + 2 * m.groups * m.state + m.heads, W)), (p + "mix.conv", (m.conv_channels, m.conv)),
+                    (p + "mix.conv.b", (m.conv_channels,)), (p + "mix.dt_bias", (m.heads,)), (p + "mix.A_log", (m.heads,)),
+                    (p + "mix.D", (m.heads,)), (p + "mix.norm", (m.inner,)), (p + "mix.o", (W, m.inner))]
+        if ml is None:
+            continue
+        if ml.kind == "dense":
+            out += [(p + "mlp.up", (ml.ff, W)), (p + "mlp.down", (W, ml.ff)), (p + "mlp.act", (4,))]
+        else:
+            for e in range(ml.experts):
+                out += [(p + f"mlp.e{e}.gate", (ml.ff, W)), (p + f"mlp.e{e}.up", (ml.ff, W)), (p + f"mlp.e{e}.down", (W, ml.ff))]
+            out.append((p + "mlp.router", (ml.experts, W)))
+    return out + [("final.norm", ()), ("head", (cfg.vocab_size, W))]
+
+
 def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
     if cfg.family == "eagle3":
         return eagle_param_shapes(cfg)
@@ -110,6 +145,8 @@ def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
         return fatulix_param_shapes(cfg)
     if cfg.family == "zerusun":
         return zerusun_param_shapes(cfg)
+    if cfg.family == "fomunex":
+        return fomunex_param_shapes(cfg)
     h, hd, nh, nkv, I, V = cfg.hidden_size, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, cfg.intermediate_size, cfg.vocab_size
     out = [("model.embed_tokens.weight", (V, h))]
     for i in range(cfg.num_layers):
