@@ -514,14 +514,15 @@ int ssd_moe_route_sigmoid(const float* logits, long ld, int32_t* idx, float* wei
  * K cache [blocks][G][block_size][D] row slots[t] (-1: none) = k / rms(k); V cache [blocks][G][Dv][block_size] (transposed per page).
  * Attention: out[t][h] (Dv wide) = sum_j p_j v_j over the keys j of the token's sequence with 0 <= positions[t] - j < window
  * (window 0: all keys up to the token), s_j = cap * tanh(scale * <q, k_j> / cap) - slopes[h] * (positions[t] - j) (cap <= 0: no cap;
- * slopes NULL: no penalty), p_j = exp(s_j) / (sum_j' exp(s_j') + exp(sinks[h])) (sinks NULL: no sink).  workspace (optional, fp32):
- * with few rows the MFMA form cuts the window into key slices over the grid and merges them. */
+ * slopes NULL: no penalty), p_j = exp(s_j) / (sum_j' exp(s_j') + exp(sinks[h])) (sinks NULL: no sink).  max_q > 0 (an upper bound of
+ * the rows any sequence of the batch brings) admits the MFMA form for bf16 and D % 32 == 0, Dv % 16 == 0, block_size % 32 == 0; max_q = 0
+ * or other sizes or fp32: the scalar form. */
 int ssd_winattn_store(const void* qkv_rows, long ld, float eps, const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int T,
                       int H, int G, int D, int Dv, int block_size, int f32, void* stream);
 int ssd_winattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const float* slopes, const float* sinks,
-                      const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B,
-                      int T, int H, int G, int D, int Dv, int block_size, int window, float scale, float cap, void* out_rows, int f32,
-                      void* stream);
+                      const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq,
+                      int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, int window, float scale, float cap,
+                      void* out_rows, int f32, void* stream);
 
 /* Recurrent mixers over per-sequence state slots (csrc/recurrent.hip).  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows
  * each; state_slots int32 [B]; a sequence whose first row has position 0 starts from zero whatever its slot holds.

@@ -21,10 +21,6 @@ def scalar_norm(x, g, eps):
     return rms(x, eps) * g.to(F64).reshape(())
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def silu(z):
     return z * torch.sigmoid(z)
 
@@ -173,3 +169,128 @@ def forward(cfg: dict, w: dict, tokens, taps: list | None = None, round_input=No
     logits = lin(w["head"], scalar_norm(x, w["final.norm"], eps)) * float(cfg.get("logit_scale", 1.0))
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# configurations and random weights for tests
+# ------------------------------------------------------------------------------------------------------------------
+def dense_mlp(ff: int = 40) -> dict:
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_mlp(experts: int = 5, top: int = 2, ff: int = 24, limit: float = 1.5) -> dict:
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
+
+
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=24, scale=0.6, softcap=12.0, window=9, mlp=None, weights_of=None) -> dict:
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if softcap:
+        m["softcap"] = softcap
+    if window:
+        m["mask"] = {"size": window}
+    out = {"type": "attention", "mixer": m, "mlp": mlp}
+    if weights_of is not None:
+        out["weights_of"] = weights_of
+    return out
+
+
+def wkv_layer(heads=3, dim=8, decay_rank=6, mlp=None, weights_of=None) -> dict:
+    """decay_rank is not a config.json key (the checkpoint's tensor shapes give it); random_model reads it from here and drops it."""
+    out = {"type": "wkv", "mixer": {"heads": heads, "dim": dim, "decay_rank": decay_rank}, "mlp": mlp}
+    if weights_of is not None:
+        out["weights_of"] = weights_of
+    return out
+
+
+def mamba2_layer(heads=4, vdim=12, state=8, groups=2, conv=4, norm_groups=2, mlp=None, weights_of=None) -> dict:
+    out = {"type": "mamba2", "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv, "norm_groups": norm_groups},
+           "mlp": mlp}
+    if weights_of is not None:
+        out["weights_of"] = weights_of
+    return out
+
+
+def make_config(layers, vocab=97, width=48, eps=1e-5, max_positions=512, logit_scale=1.5, logit_softcap=25.0) -> dict:
+    cfg = {"architecture": "Fomunex", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": eps}, "layers": layers}
+    if logit_scale is not None:
+        cfg["logit_scale"] = logit_scale
+    if logit_softcap:
+        cfg["logit_softcap"] = logit_softcap
+    return cfg
+
+
+def random_model(cfg: dict, seed: int = 0, keep_rank: bool = False) -> dict:
+    """bf16 weights of the right shapes for `cfg`: matrices N(0, 1 / fan-in), norm numbers around 1, decays that remember hundreds of
+    tokens in some channels and a few in others.  Unless keep_rank, the layers' decay_rank entries are removed from cfg afterwards (a
+    checkpoint's tensor shapes carry that size)."""
+    gen = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    w = {}
+    bf = torch.bfloat16
+
+    def mat(name, o, i, gain=1.0):
+        w[name] = (torch.randn(o, i, generator=gen) * gain / math.sqrt(i)).to(bf)
+
+    def vec(name, n, base=1.0, s=0.1):
+        w[name] = (base + s * torch.randn(n, generator=gen)).to(bf)
+
+    def uni(name, n, lo, hi):
+        w[name] = (lo + (hi - lo) * torch.rand(n, generator=gen)).to(bf)
+
+    def scalar(name):
+        w[name] = torch.tensor(0.8 + 0.5 * torch.rand((), generator=gen).item()).to(bf)
+
+    mat("embed", cfg["vocab"], W, math.sqrt(W))
+    w["pos"] = (0.5 * torch.randn(cfg["max_positions"], W, generator=gen)).to(bf)
+    for i, lc in enumerate(cfg["layers"]):
+        if lc.get("weights_of", i) != i:
+            continue
+        p, m, ml = f"l{i}.", lc["mixer"], lc.get("mlp")
+        scalar(p + "norm1")
+        if lc["type"] == "attention":
+            mat(p + "mix.q", m["heads"] * m["dim"], W, 2.0)
+            mat(p + "mix.k", m["kv_heads"] * m["dim"], W, 2.0)
+            mat(p + "mix.v", m["kv_heads"] * m["vdim"], W)
+            vec(p + "mix.sink", m["heads"], 0.0, 1.5)
+            mat(p + "mix.o", W, m["heads"] * m["vdim"])
+        elif lc["type"] == "wkv":
+            n, R = m["heads"] * m["dim"], m["decay_rank"]
+            for s in "rkvgw":
+                uni(p + "mix.mu." + s, W, 0.0, 1.0)
+            for s in "rkvg":
+                mat(p + "mix." + s, n, W, 1.5)
+            mat(p + "mix.w1", R, W)
+            mat(p + "mix.w2", n, R)
+            uni(p + "mix.w0", n, -6.0, 0.5)
+            w[p + "mix.u"] = (0.5 * torch.randn(m["heads"], m["dim"], generator=gen)).to(bf)
+            vec(p + "mix.norm", n)
+            mat(p + "mix.o", W, n)
+        else:
+            inner, C = m["heads"] * m["vdim"], m["heads"] * m["vdim"] + 2 * m["groups"] * m["state"]
+            mat(p + "mix.in", 2 * inner + 2 * m["groups"] * m["state"] + m["heads"], W, 1.5)
+            w[p + "mix.conv"] = (torch.randn(C, m["conv"], generator=gen) / math.sqrt(m["conv"])).to(bf)
+            vec(p + "mix.conv.b", C, 0.0, 0.2)
+            uni(p + "mix.dt_bias", m["heads"], -4.0, 0.5)
+            uni(p + "mix.A_log", m["heads"], -3.0, 1.0)
+            vec(p + "mix.D", m["heads"], 0.5, 0.5)
+            vec(p + "mix.norm", inner)
+            mat(p + "mix.o", W, inner)
+        if ml is None:
+            continue
+        scalar(p + "norm2")
+        if ml["kind"] == "dense":
+            mat(p + "mlp.up", ml["ff"], W, 1.5)
+            mat(p + "mlp.down", W, ml["ff"])
+            w[p + "mlp.act"] = torch.tensor([0.9, 0.4, -0.3, 0.1]).add(0.1 * torch.randn(4, generator=gen)).to(bf)
+        else:
+            for e in range(ml["router"]["experts"]):
+                mat(p + f"mlp.e{e}.gate", ml["expert"]["ff"], W, 2.5)
+                mat(p + f"mlp.e{e}.up", ml["expert"]["ff"], W, 2.5)
+                mat(p + f"mlp.e{e}.down", W, ml["expert"]["ff"])
+            mat(p + "mlp.router", ml["router"]["experts"], W, 2.0)
+    scalar("final.norm")
+    mat("head", cfg["vocab"], W, 2.0)
+    if not keep_rank:
+        for lc in cfg["layers"]:
+            lc["mixer"].pop("decay_rank", None)
+    return w

@@ -11,7 +11,8 @@
 //                         the window's first key (so a row's summation order is a function of its own position only); a lane owns a
 //                         KEY for the scores and a VALUE COLUMN for the sums; partial (max, sum, accumulator) triples merge in LDS in
 //                         wave order, then the sink joins the denominator.
-//                         MFMA form (bf16, D % 32 == 0, D <= 256, Dv % 16 == 0, Dv <= 256, block_size % 32 == 0): see below.
+//                         MFMA form (bf16, D % 32 == 0, D <= 256, Dv % 16 == 0, Dv <= 256, block_size % 32 == 0; the caller gives
+//                         max_q, an upper bound of the rows a sequence brings): see below.
 //   Scores, weights, sums and norms are fp32 whatever the element type.  A token's position and sequence come from positions[] and
 //   cu_q[] (varlen batches: prompt portions beside single tokens) or q_per_seq (fixed rows per sequence).
 #include "common.h"
@@ -159,6 +160,194 @@ winattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T*
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// MFMA form (bf16, D % 32 == 0, D <= 256, Dv % 16 == 0, Dv <= 256, block_size % 32 == 0).  For one kv head, the query ROWS of a
+// sequence are its (token, head of the group) pairs, token-major; a wave owns 16 rows and walks the keys in steps of 32 that start
+// at multiples of 32 of the key index (never across a page):
+//   S[key][row]  = K tile (A operand: cache rows as they lie) x Q (B operand, in registers), two 16-key tiles per step, fp32
+//   cap, distance penalty, window and causal mask (by select: whatever the cache holds at a masked key cannot leak), online
+//   softmax per row in fp32 on the accumulator fragments (a lane holds 8 keys of one row; a row's 4 lanes meet by two shuffles)
+//   O[dv][row]  += V^T tile (A operand: two 8-byte loads from the transposed page) x P (B operand: the lane's 8 weights as bf16);
+//   the k slots of the second product are the keys in the order the first product's fragments hold them: no data moves between lanes.
+// tile mode  (a sequence brings more than 16 rows): workgroup = 4 waves = 64 consecutive rows; every wave walks the keys from the
+//            window start of its first row to the position of its last.
+// split mode (<= 16 rows: decoding): the 4 waves share the rows and take the steps round-robin; partial (max, sum, O) meet in LDS and
+//            are merged in wave order.  The window bounds the steps, so the keys are not cut over the grid.
+// V of keys past the last row's position is zeroed (a weight of zero times whatever an unwritten slot holds must stay zero).
+// The sink joins the denominator at the end.  The cap's tanh is 1 - 2 / (1 + exp(2x)) on the fast exponential.
+// ---------------------------------------------------------------------------------------------------------------------
+template <int MK, int MV>        // upper bounds of D / 32 and Dv / 16 (register arrays)
+__global__ void __launch_bounds__(256)
+winattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vt,
+                    const float* __restrict__ slopes, const float* __restrict__ sinks, const int32_t* __restrict__ bt, int max_blocks,
+                    const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq, int H, int G, int D, int Dv,
+                    int bs, int window, float scale, float cap, bf16_t* __restrict__ out) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
+  const int b = blockIdx.z, g = blockIdx.y, R = H / G;
+  const int KS = D >> 5, DVT = Dv >> 4;
+  const int tok0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int nrows = (cu_q ? cu_q[b + 1] - tok0 : q_per_seq) * R;
+  const bool split = nrows <= 16;
+  if ((int)blockIdx.x * 64 >= nrows) return;
+  const int row0 = split ? 0 : blockIdx.x * 64 + wave * 16;
+  if (!split && row0 >= nrows) return;                 // (tile mode has no workgroup barriers)
+  const int row = row0 + r;
+  const bool valid = row < nrows;
+  const int rr = valid ? row : row0;
+  const int token = tok0 + rr / R, head = g * R + rr % R;
+  const int pos = valid ? (int)positions[token] : -1;
+  const int first = valid ? (window > 0 && pos + 1 > window ? pos + 1 - window : 0) : 0x7fffffff;
+  const float slope = slopes ? slopes[head] : 0.f;
+  int kmax = pos, kmin = first;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { kmax = max(kmax, __shfl_xor(kmax, o, 64)); kmin = min(kmin, __shfl_xor(kmin, o, 64)); }
+  const int32_t* table = bt + (size_t)b * max_blocks;
+
+  u32x4_t qreg[MK];
+  const bf16_t* qrow = q + ((size_t)token * H + head) * D;
+#pragma unroll
+  for (int ks = 0; ks < MK; ++ks) {
+    qreg[ks] = u32x4_t{0u, 0u, 0u, 0u};
+    if (ks < KS && valid) qreg[ks] = *reinterpret_cast<const u32x4_t*>(qrow + ks * 32 + qd * 8);
+  }
+  float mx = -INFINITY, ls = 0.f;
+  f32x4_t acc[MV];
+#pragma unroll
+  for (int i = 0; i < MV; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const float inv_cap = cap > 0.f ? 1.0f / cap : 0.f;
+
+  const int s_first = kmin >> 5, s_last = kmax >> 5;
+  for (int st = s_first + (split ? wave : 0); st <= s_last; st += split ? 4 : 1) {
+    const int k0 = st << 5;
+    const size_t pg = (size_t)table[k0 / bs] * G + g;
+    const int koff = k0 % bs;
+    u32x4_t kreg[2][MK];
+    u32x2_t vlo[MV], vhi[MV];
+#pragma unroll
+    for (int hg = 0; hg < 2; ++hg) {
+      const bf16_t* kr = kc + (pg * bs + koff + hg * 16 + r) * D + qd * 8;
+#pragma unroll
+      for (int ks = 0; ks < MK; ++ks) {
+        kreg[hg][ks] = u32x4_t{0u, 0u, 0u, 0u};
+        if (ks < KS) kreg[hg][ks] = *reinterpret_cast<const u32x4_t*>(kr + ks * 32);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < MV; ++i) {
+      vlo[i] = u32x2_t{0u, 0u};
+      vhi[i] = u32x2_t{0u, 0u};
+      if (i < DVT) {
+        const bf16_t* vp = vt + (pg * Dv + i * 16 + r) * bs + koff + qd * 4;
+        vlo[i] = *reinterpret_cast<const u32x2_t*>(vp);
+        vhi[i] = *reinterpret_cast<const u32x2_t*>(vp + 16);
+      }
+    }
+    if (k0 + 31 > kmax) {       // keys past the last row's position were never stored: whatever lies there must not meet a zero weight
+      const int ka = k0 + qd * 4;
+      const uint32_t l0 = (ka <= kmax ? 0xffffu : 0u) | (ka + 1 <= kmax ? 0xffff0000u : 0u);
+      const uint32_t l1 = (ka + 2 <= kmax ? 0xffffu : 0u) | (ka + 3 <= kmax ? 0xffff0000u : 0u);
+      const uint32_t h0 = (ka + 16 <= kmax ? 0xffffu : 0u) | (ka + 17 <= kmax ? 0xffff0000u : 0u);
+      const uint32_t h1 = (ka + 18 <= kmax ? 0xffffu : 0u) | (ka + 19 <= kmax ? 0xffff0000u : 0u);
+#pragma unroll
+      for (int i = 0; i < MV; ++i) { vlo[i][0] &= l0; vlo[i][1] &= l1; vhi[i][0] &= h0; vhi[i][1] &= h1; }
+    }
+    f32x4_t sc[2];
+#pragma unroll
+    for (int hg = 0; hg < 2; ++hg) {
+      sc[hg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < MK; ++ks)
+        if (ks < KS) sc[hg] = mfma16(kreg[hg][ks], qreg[ks], sc[hg]);
+    }
+    // lane (row r, keys k0 + hg * 16 + qd * 4 + i)
+    float sv[8], smax = -INFINITY;
+#pragma unroll
+    for (int hg = 0; hg < 2; ++hg)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + hg * 16 + qd * 4 + i;
+        float s = sc[hg][i] * scale;
+        if (cap > 0.f) s = cap * (1.0f - 2.0f / (1.0f + __expf(2.0f * s * inv_cap)));
+        s -= slope * (float)(pos - key);
+        s = (key <= pos && key >= first) ? s : -INFINITY;
+        sv[hg * 4 + i] = s;
+        smax = fmaxf(smax, s);
+      }
+    smax = fmaxf(smax, __shfl_xor(smax, 16, 64));
+    smax = fmaxf(smax, __shfl_xor(smax, 32, 64));
+    const float mn = fmaxf(mx, smax);
+    const float c = mn == -INFINITY ? 1.0f : __expf(mx - mn);
+    float psum = 0.f, pv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      pv[i] = sv[i] == -INFINITY ? 0.f : __expf(sv[i] - mn);
+      psum += pv[i];
+    }
+    ls = ls * c + psum;
+    mx = mn;
+    u32x4_t pb;
+    pb[0] = pack_bf2_hw(pv[0], pv[1]); pb[1] = pack_bf2_hw(pv[2], pv[3]);
+    pb[2] = pack_bf2_hw(pv[4], pv[5]); pb[3] = pack_bf2_hw(pv[6], pv[7]);
+#pragma unroll
+    for (int i = 0; i < MV; ++i)
+      if (i < DVT) {
+        acc[i] *= c;
+        const u32x4_t va = u32x4_t{vlo[i][0], vlo[i][1], vhi[i][0], vhi[i][1]};
+        acc[i] = mfma16(va, pb, acc[i]);
+      }
+  }
+  ls += __shfl_xor(ls, 16, 64);
+  ls += __shfl_xor(ls, 32, 64);
+
+  if (split) {
+    // partial rows of the four waves meet in LDS: [wave][16 rows][Dv] sums, [wave][16] max and sum; merged in wave order
+    float* so = smem;                               // [4][16][Dv]
+    float* sm = so + 4 * 16 * Dv;                   // [4][16]
+    float* sl = sm + 64;                            // [4][16]
+#pragma unroll
+    for (int i = 0; i < MV; ++i)
+      if (i < DVT)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) so[(wave * 16 + r) * Dv + i * 16 + qd * 4 + e] = acc[i][e];
+    if (qd == 0) { sm[wave * 16 + r] = mx; sl[wave * 16 + r] = ls; }
+    __syncthreads();
+    if (wave != 0) return;
+    float M = -INFINITY;
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, sm[w * 16 + r]);
+    float f[4], L = 0.f;
+    for (int w = 0; w < 4; ++w) {
+      f[w] = sl[w * 16 + r] > 0.f ? __expf(sm[w * 16 + r] - M) : 0.f;
+      L += sl[w * 16 + r] * f[w];
+    }
+#pragma unroll
+    for (int i = 0; i < MV; ++i)
+      if (i < DVT)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float o = 0.f;
+          for (int w = 0; w < 4; ++w) o += so[(w * 16 + r) * Dv + i * 16 + qd * 4 + e] * f[w];
+          acc[i][e] = o;
+        }
+    mx = M; ls = L;
+  }
+  if (!valid) return;
+  const float sink = sinks ? sinks[head] : -INFINITY;
+  const float M = fmaxf(mx, sink);
+  const float fo = ls > 0.f ? __expf(mx - M) : 0.f;
+  const float den = ls * fo + (sinks ? __expf(sink - M) : 0.f);
+  const float rs = fo / den;
+  bf16_t* orow = out + ((size_t)token * H + head) * Dv + qd * 4;
+#pragma unroll
+  for (int i = 0; i < MV; ++i)
+    if (i < DVT) {
+      u32x2_t o2;
+      o2[0] = pack_bf2_hw(acc[i][0] * rs, acc[i][1] * rs);
+      o2[1] = pack_bf2_hw(acc[i][2] * rs, acc[i][3] * rs);
+      *reinterpret_cast<u32x2_t*>(orow + i * 16) = o2;
+    }
+}
+
 }  // namespace
 
 #define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
@@ -181,12 +370,31 @@ extern "C" int ssd_winattn_store(const void* qkv_rows, long ld, float eps, const
 
 extern "C" int ssd_winattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const float* slopes, const float* sinks,
                                  const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q,
-                                 int q_per_seq, int B, int T, int H, int G, int D, int Dv, int block_size, int window, float scale,
-                                 float cap, void* out_rows, int f32, void* stream) {
+                                 int q_per_seq, int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, int window,
+                                 float scale, float cap, void* out_rows, int f32, void* stream) {
   if (!q_rows || !k_cache || !v_cache || !block_tables || !positions || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * WA_MAXV || block_size <= 0 || window < 0 ||
       max_blocks <= 0 || (!cu_q && q_per_seq <= 0) || H > 65535)
     return SSD_ERR_SHAPE;
+  if (!f32 && max_q > 0 && D % 32 == 0 && D <= 256 && Dv % 16 == 0 && Dv <= 256 && block_size % 32 == 0 && G <= 65535 && B <= 65535) {
+    const int R = H / G;
+    const dim3 grid((unsigned)(((long)max_q * R + 63) / 64), G, B);
+    const size_t lds = (4 * 16 * (size_t)Dv + 128) * sizeof(float);
+#define WIN_MFMA(MK, MV)                                                                                                            \
+  hipLaunchKernelGGL((winattn_mfma_kernel<MK, MV>), grid, dim3(256), lds, (hipStream_t)stream, (const bf16_t*)q_rows,               \
+                     (const bf16_t*)k_cache, (const bf16_t*)v_cache, slopes, sinks, block_tables, max_blocks, positions, cu_q,      \
+                     q_per_seq, H, G, D, Dv, block_size, window, scale, cap, (bf16_t*)out_rows)
+    if (D <= 64 && Dv <= 64) WIN_MFMA(2, 4);
+    else if (D <= 128 && Dv <= 128) WIN_MFMA(4, 8);
+    else {
+      if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)winattn_mfma_kernel<8, 16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 (int)lds) != hipSuccess)
+        return SSD_ERR_LAUNCH;
+      WIN_MFMA(8, 16);
+    }
+#undef WIN_MFMA
+    return LAUNCH_OK();
+  }
   const size_t bytes = ((size_t)D + (D & 1) + 4 * 64 + 2 * 4 * 64 + 4 * (size_t)Dv + 8) * sizeof(float);
   if (bytes > 64 * 1024) return SSD_ERR_SHAPE;
   if (f32)

@@ -156,6 +156,28 @@ causal_conv_silu_kernel(const float* __restrict__ proj, long ld, int col_off, in
 
 constexpr int CONV_MAX_TAPS = 16;
 
+__device__ __forceinline__ void save_conv_state(const float* proj, long ld, int conv_off, int C, float* conv_state, int taps, int slot,
+                                                int row0, int row1, long p0) {
+  const int n = row1 - row0, K1 = taps - 1;
+  float* st = conv_state + (size_t)slot * K1 * C;
+  for (int c = threadIdx.x; c < C; c += 256) {
+    float keep[CONV_MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS; ++i) {
+      keep[i] = 0.f;
+      if (i < K1) {
+        const long rel = (long)n - K1 + i;                // position relative to the portion's first row
+        if (rel >= 0) keep[i] = proj[(size_t)(row0 + rel) * ld + conv_off + c];
+        else if (p0 + rel >= 0) keep[i] = st[(size_t)(i + n) * C + c];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS; ++i)
+      if (i < K1) st[(size_t)i * C + c] = keep[i];
+  }
+}
+
+
 __global__ void __launch_bounds__(256)
 ssd_scan_kernel(const float* __restrict__ xbc, long ldx, int x_off, int b_off, int c_off, const float* __restrict__ proj, long ld,
                 int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ dskip,
@@ -196,24 +218,111 @@ ssd_scan_kernel(const float* __restrict__ xbc, long ldx, int x_off, int b_off, i
   }
   __syncthreads();
   for (int i = tid; i < N * Dv; i += 256) sp[i] = S[i];
-  if (h == 0 && taps > 1) {
-    // the slot's last taps - 1 convolution inputs: saved row i holds the input of position p0 + n - (taps - 1) + i
-    const int n = row1 - row0, K1 = taps - 1;
-    float* st = conv_state + (size_t)slot * K1 * C;
-    for (int c = tid; c < C; c += 256) {
-      float keep[CONV_MAX_TAPS];
+  if (h == 0 && taps > 1)      // the slot's last taps - 1 convolution inputs: saved row i holds the input of position p0 + n - (taps - 1) + i
+    save_conv_state(proj, ld, conv_off, C, conv_state, taps, slot, row0, row1, p0);
+}
+
+// Register form of both scans (state rows D = 8 * EPT with EPT in {4, 8, 16, 32}, Dv % 32 == 0): a workgroup owns 32 state columns of one
+// (sequence, head) -- grid.z walks the column blocks -- and thread (g, e) keeps the EPT elements (d = g + 8 n, column e) in registers.
+// Rows are staged eight at a time (decays and step sizes computed once per row), every thread then walks the eight tokens without a
+// barrier, and the eight d-groups' partial outputs are summed in group order.  The arithmetic of a row is the same for any portioning:
+// the per-element chain in token order, the output sum over n ascending, then over g ascending.
+struct WkvArgs {
+  const float* proj; long ld; int r_off, k_off, v_off; const float* ww; long ldw; const float* w0; const float* u;
+};
+struct SsdArgs {
+  const float* xbc; long ldx; int x_off, b_off, c_off; const float* proj; long ld; int dt_off; const float* dt_bias; const float* a_log;
+  const float* skip; int G, conv_off, C, taps; float* conv_state;
+};
+
+template <int MODE, int EPT, typename T>
+__global__ void __launch_bounds__(256)
+scan_reg_kernel(WkvArgs wa, SsdArgs sa, const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
+                const int32_t* __restrict__ state_slots, float* __restrict__ state, float* __restrict__ out, const T* __restrict__ hn,
+                float* __restrict__ shift_state, int W, int H, int Dv) {
+  constexpr int TB = 8, NG = 8, CB = 32, D = NG * EPT;
+  __shared__ float sq[TB][D], sk[TB][D], sd[TB][MODE == 0 ? D : 1];
+  __shared__ float sv[TB][CB];
+  __shared__ float sdt[TB];
+  __shared__ float po[TB][NG][CB];
+  const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CB, tid = threadIdx.x;
+  const int g = tid >> 5, e = tid & 31;
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int row1 = cu_q ? cu_q[b + 1] : (b + 1) * q_per_seq;
+  if (row1 <= row0) return;
+  const int slot = state_slots[b];
+  float* sp = state + ((size_t)slot * H + h) * D * Dv + c0 + e;
+  const long p0 = positions[row0];
+  const bool fresh = p0 == 0;
+  float S[EPT], U[EPT];
 #pragma unroll
-      for (int i = 0; i < CONV_MAX_TAPS; ++i) {
-        keep[i] = 0.f;
-        if (i < K1) {
-          const long rel = (long)n - K1 + i;                // position relative to the portion's first row
-          if (rel >= 0) keep[i] = proj[(size_t)(row0 + rel) * ld + conv_off + c];
-          else if (p0 + rel >= 0) keep[i] = st[(size_t)(i + n) * C + c];
+  for (int n = 0; n < EPT; ++n) {
+    S[n] = fresh ? 0.f : sp[(size_t)(g + NG * n) * Dv];
+    U[n] = MODE == 0 ? wa.u[h * D + g + NG * n] : 0.f;
+  }
+  const int grp = MODE == 1 ? h / (H / sa.G) : 0;
+  const float a = MODE == 1 ? -expf(sa.a_log[h]) : 0.f, dtb = MODE == 1 ? sa.dt_bias[h] : 0.f, skip = MODE == 1 ? sa.skip[h] : 0.f;
+  for (int r = row0; r < row1; r += TB) {
+    const int nb = row1 - r < TB ? row1 - r : TB;
+    __syncthreads();                      // the previous batch's readers are done
+    if (MODE == 1) {
+      if (tid < nb) {
+        const float dt = softplusf_(sa.proj[(size_t)(r + tid) * sa.ld + sa.dt_off + h] + dtb);
+        sdt[tid] = dt;
+        sd[tid][0] = expf(a * dt);
+      }
+      __syncthreads();
+    }
+    for (int idx = tid; idx < nb * D; idx += 256) {
+      const int tt = idx / D, d = idx % D;
+      if (MODE == 0) {
+        const float* pr = wa.proj + (size_t)(r + tt) * wa.ld + h * D + d;
+        sq[tt][d] = pr[wa.r_off];
+        sk[tt][d] = pr[wa.k_off];
+        sd[tt][d] = expf(-expf(wa.ww[(size_t)(r + tt) * wa.ldw + h * D + d] + wa.w0[h * D + d]));
+      } else {
+        const float* xr = sa.xbc + (size_t)(r + tt) * sa.ldx + grp * D + d;
+        sq[tt][d] = xr[sa.c_off];
+        sk[tt][d] = sdt[tt] * xr[sa.b_off];
+      }
+    }
+    if (g < nb)
+      sv[g][e] = MODE == 0 ? wa.proj[(size_t)(r + g) * wa.ld + wa.v_off + h * Dv + c0 + e]
+                           : sa.xbc[(size_t)(r + g) * sa.ldx + sa.x_off + h * Dv + c0 + e];
+    __syncthreads();
+    for (int tt = 0; tt < nb; ++tt) {
+      const float ve = sv[tt][e];
+      float o = 0.f;
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) {
+        const int d = g + NG * n;
+        const float kv = sk[tt][d] * ve;
+        if (MODE == 0) {
+          o = fmaf(fmaf(U[n], kv, S[n]), sq[tt][d], o);
+          S[n] = fmaf(sd[tt][d], S[n], kv);
+        } else {
+          S[n] = fmaf(sd[tt][0], S[n], kv);
+          o = fmaf(S[n], sq[tt][d], o);
         }
       }
+      po[tt][g][e] = o;
+    }
+    __syncthreads();
+    if (g < nb) {                         // thread (g, e) now finishes token g of the batch
+      float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < CONV_MAX_TAPS; ++i)
-        if (i < K1) st[(size_t)i * C + c] = keep[i];
+      for (int gg = 0; gg < NG; ++gg) o += po[g][gg][e];
+      if (MODE == 1) o = fmaf(skip, sv[g][e], o);
+      out[(size_t)(r + g) * H * Dv + h * Dv + c0 + e] = o;
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < EPT; ++n) sp[(size_t)(g + NG * n) * Dv] = S[n];
+  if (h == 0 && blockIdx.z == 0) {
+    if (MODE == 0) {
+      for (int c = tid; c < W; c += 256) shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
+    } else if (sa.taps > 1) {
+      save_conv_state(sa.proj, sa.ld, sa.conv_off, sa.C, sa.conv_state, sa.taps, slot, row0, row1, p0);
     }
   }
 }
@@ -273,6 +382,27 @@ extern "C" int ssd_wkv_scan(const void* proj_rows, long ld, int r_off, int k_off
   if (!proj_rows || !decay_rows || !w0 || !u || !positions || !state_slots || !state || !out_rows || !hn_rows || !shift_state)
     return SSD_ERR_ARG;
   if (B <= 0 || H <= 0 || D <= 0 || W <= 0 || (!cu_q && q_per_seq <= 0) || H > 65535) return SSD_ERR_SHAPE;
+  if (D % 32 == 0 && (D == 32 || D == 64 || D == 128 || D == 256)) {
+    const WkvArgs wa{(const float*)proj_rows, ld, r_off, k_off, v_off, (const float*)decay_rows, ldw, w0, u};
+    const SsdArgs sa{};
+    const dim3 grid(B, H, D / 32);
+#define WKV_REG(EPT)                                                                                                                 \
+  do {                                                                                                                               \
+    if (f32)                                                                                                                         \
+      hipLaunchKernelGGL((scan_reg_kernel<0, EPT, float>), grid, dim3(256), 0, (hipStream_t)stream, wa, sa, positions, cu_q, q_per_seq, \
+                         state_slots, (float*)state, (float*)out_rows, (const float*)hn_rows, (float*)shift_state, W, H, D);        \
+    else                                                                                                                             \
+      hipLaunchKernelGGL((scan_reg_kernel<0, EPT, bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, wa, sa, positions, cu_q,        \
+                         q_per_seq, state_slots, (float*)state, (float*)out_rows, (const bf16_t*)hn_rows, (float*)shift_state, W, H, \
+                         D);                                                                                                         \
+  } while (0)
+    if (D == 32) WKV_REG(4);
+    else if (D == 64) WKV_REG(8);
+    else if (D == 128) WKV_REG(16);
+    else WKV_REG(32);
+#undef WKV_REG
+    return LAUNCH_OK();
+  }
   const int EP = pick_ep(D);
   const size_t bytes = ((size_t)D * D + 6 * (size_t)D + (size_t)(256 / EP) * D) * sizeof(float);
   if (bytes > 160 * 1024) return SSD_ERR_SHAPE;
@@ -317,6 +447,21 @@ extern "C" int ssd_ssd_scan(const void* xbc_rows, long ldx, int x_off, int b_off
   if (B <= 0 || H <= 0 || G <= 0 || H % G || N <= 0 || Dv <= 0 || taps < 1 || taps > CONV_MAX_TAPS || C <= 0 ||
       (!cu_q && q_per_seq <= 0) || H > 65535)
     return SSD_ERR_SHAPE;
+  if (Dv % 32 == 0 && Dv / 32 <= 65535 && (N == 32 || N == 64 || N == 128 || N == 256)) {
+    const WkvArgs wa{};
+    const SsdArgs sa{(const float*)xbc_rows, ldx, x_off, b_off, c_off, (const float*)proj_rows, ld, dt_off, dt_bias, a_log, skip, G,
+                     conv_off, C, taps, (float*)conv_state};
+    const dim3 grid(B, H, Dv / 32);
+#define SSD_REG(EPT)                                                                                                               \
+  hipLaunchKernelGGL((scan_reg_kernel<1, EPT, float>), grid, dim3(256), 0, (hipStream_t)stream, wa, sa, positions, cu_q, q_per_seq, \
+                     state_slots, (float*)state, (float*)out_rows, (const float*)nullptr, (float*)nullptr, 0, H, Dv)
+    if (N == 32) SSD_REG(4);
+    else if (N == 64) SSD_REG(8);
+    else if (N == 128) SSD_REG(16);
+    else SSD_REG(32);
+#undef SSD_REG
+    return LAUNCH_OK();
+  }
   const int EP = pick_ep(Dv);
   const size_t bytes = ((size_t)N * Dv + 3 * (size_t)N + Dv + (size_t)(256 / EP) * Dv) * sizeof(float);
   if (bytes > 160 * 1024) return SSD_ERR_SHAPE;

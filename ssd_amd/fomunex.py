@@ -55,6 +55,7 @@ class HipFomunex(Res32Decoder):
         self.w: dict[str, torch.Tensor] = {}
         self.kv: list = []
         self.state: list = []
+        self.scalar_attention = False                 # tests / probes: the scalar form of the attention also where the MFMA form fits
         self.tap_residuals: list | None = None         # tests: receives a copy of the residual rows after every layer (eager only)
 
         def z(*shape, dtype=torch.float32):
@@ -237,7 +238,7 @@ class HipFomunex(Res32Decoder):
             H.winattn_store(self.proj, NP, cfg.rms_norm_eps, meta.slot_mapping, self.q, kc, vc, T, m.heads, m.kv_heads, m.dim, m.vdim,
                             self.block_size, f)
             H.winattn_paged(self.q, kc, vc, w[p + "slopes"], w[p + "sink"], meta.block_tables, self.max_blocks, positions, meta.B, T,
-                            m.heads, m.kv_heads, m.dim, m.vdim, self.block_size, m.window, m.scale, m.softcap, self.att, f, **seqs)
+                            m.heads, m.kv_heads, m.dim, m.vdim, self.block_size, m.window, m.scale, m.softcap, self.att, f, max_q=0 if self.scalar_attention else meta.max_q, **seqs)
             n_out = m.heads * m.vdim
         elif m.kind == "wkv":
             assert meta.state_slots is not None, "a model with recurrent layers needs the sequences' state slots"

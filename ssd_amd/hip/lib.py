@@ -151,7 +151,7 @@ SIGNATURES = {
     "ssd_moe_route_sigmoid": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_winattn_store": [c_void_p, c_long, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
-    "ssd_winattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+    "ssd_winattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p],
     "ssd_token_shift_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
                             c_int, c_void_p],

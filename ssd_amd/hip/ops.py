@@ -563,9 +563,11 @@ def winattn_store(qkv, ld: int, eps: float, slots, q_out, k_cache, v_cache, T: i
 
 
 def winattn_paged(q, k_cache, v_cache, slopes, sinks, block_tables, max_blocks: int, positions, B: int, T: int, H: int, G: int, D: int,
-                  Dv: int, block_size: int, window: int, scale: float, cap: float, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0):
+                  Dv: int, block_size: int, window: int, scale: float, cap: float, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0,
+                  max_q: int = 0):
+    """max_q > 0 (an upper bound of the rows a sequence brings; bf16, aligned head sizes, block_size % 32 == 0): the MFMA form."""
     _check(load_library().ssd_winattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(slopes), _p(sinks), _p(block_tables), max_blocks,
-                                            _p(positions), _p(cu_q), q_per_seq, B, T, H, G, D, Dv, block_size, window, scale, cap,
+                                            _p(positions), _p(cu_q), q_per_seq, max_q, B, T, H, G, D, Dv, block_size, window, scale, cap,
                                             _p(out_rows), int(f32), _stream()), "ssd_winattn_paged")
 
 

@@ -1,0 +1,358 @@
+"""The Fomunex decoder through the engine (Config -> ModelRunner -> block manager with state slots -> HIP kernels) against the plain
+whole-sequence oracle (oracle/fomunex.py, float64): small self-made configurations with random weights.  The fp32 element mode is the
+sharp one: a dropped or extra key at a window's edge, a wrong page, a lost or stale recurrent state, a forgotten sink or a missed
+convolution input is orders of magnitude above rounding there.  Attention scales are chosen so that single keys carry the output, and
+the decays so that some channels remember hundreds of tokens."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import fomunex as F
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+
+
+def write_model(path, cfg, w):
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(path, "model.safetensors"))
+    return str(path)
+
+
+def row_err(got: torch.Tensor, ref: torch.Tensor) -> torch.Tensor:
+    d = got.double().cpu() - ref.double()
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / ref.double().std()
+
+
+def rel_err(got, ref) -> float:
+    return float(row_err(got, ref).max())
+
+
+def close(got, ref, dtype) -> bool:
+    """fp32: every position within 1e-4 of the spread.  bf16: rounding of GEMM inputs, and now and then a router decision made the other
+    way at a near-tie, which in these tiny models (a few experts, a few values wide) moves that position by tens of percent: the median
+    within 5 %, nine positions in ten within 20 %, all finite.  What a schedule, the cache or the state could get wrong is pinned by
+    the fp32 runs."""
+    e = row_err(got, ref)
+    if dtype == "float32":
+        return bool(e.max() < TOL[dtype])
+    return bool(torch.isfinite(got).all() and e.median() < 0.05 and e.quantile(0.9) < 0.2)
+
+
+def configs():
+    A, K, S, D, M = F.attention_layer, F.wkv_layer, F.mamba2_layer, F.dense_mlp, F.moe_mlp
+    return {
+        # every mixer and feed-forward, two layers that borrow weights (with memory of their own); sizes chosen so that nothing the
+        # kernels index by coincides
+        "all_kinds": F.make_config([A(mlp=D()), K(mlp=M()), S(mlp=D(56)),
+                                    A(heads=3, kv_heads=1, dim=24, vdim=8, scale=0.9, softcap=0, window=33, mlp=M(experts=6, top=3, ff=16)),
+                                    A(weights_of=0, mlp=D()), K(weights_of=1, mlp=M()), S(weights_of=2, mlp=D(56))], vocab=101, width=72),
+        # values that are 1: heads, kv heads, window, experts' top, groups, norm groups, convolution taps (no saved inputs at all), logit scale
+        "ones": F.make_config([A(heads=1, kv_heads=1, dim=8, vdim=8, window=1, mlp=M(experts=3, top=1, ff=8)),
+                               K(heads=1, dim=16, decay_rank=1, mlp=D(8)), S(heads=1, vdim=8, state=8, groups=1, conv=1, norm_groups=1)],
+                              vocab=33, width=40, logit_scale=None, logit_softcap=0),
+        # no window at all, a window larger than any sequence here, every expert chosen, sizes that are no multiple of 8, no feed-forward
+        "odd_sizes": F.make_config([A(heads=6, kv_heads=3, dim=12, vdim=10, window=0, mlp=M(experts=3, top=3, ff=20, limit=0.7)),
+                                    K(heads=5, dim=12, decay_rank=3), S(heads=6, vdim=10, state=6, groups=3, conv=2, norm_groups=3, mlp=D(52)),
+                                    A(heads=2, kv_heads=2, dim=20, vdim=36, window=1000, softcap=3.0)], vocab=77, width=50, logit_scale=0.5),
+        # sizes the bf16 fast forms take (MFMA attention: head sizes in multiples of 32 / 16, more rows per token than a tile holds, one
+        # row per token; register scans: state rows 32 / 64), windows of several 32-key steps
+        "fast_forms": F.make_config([A(heads=8, kv_heads=2, dim=32, vdim=16, window=70, mlp=D(48)), K(heads=2, dim=32, mlp=M(experts=4)),
+                                     S(heads=2, vdim=32, state=32, groups=1, mlp=D(48)), A(heads=20, kv_heads=1, dim=32, vdim=32, window=0),
+                                     A(heads=4, kv_heads=4, dim=64, vdim=64, window=40, softcap=0), K(heads=1, dim=64),
+                                     S(heads=4, vdim=64, state=64, groups=2, conv=3, mlp=M(experts=4, top=1))], vocab=120, width=96),
+        # one kind of memory only: no state slots at all / no cache pages at all
+        "only_attention": F.make_config([A(window=6, mlp=M(experts=4)), A(heads=2, kv_heads=1, window=0, mlp=None)], vocab=40, width=48),
+        "only_recurrent": F.make_config([K(mlp=D()), S(mlp=M(experts=2, top=1)), K(heads=2, dim=24, weights_of=None)], vocab=40, width=48),
+    }
+
+
+def make(name, seed=0):
+    cfg = json.loads(json.dumps(configs()[name]))
+    return cfg, F.random_model(cfg, seed)
+
+
+def engine(tmp_path, cfg, w, dtype, max_tokens=512, block_size=16, **kw):
+    from ssd_amd.engine.trace_engine import TraceEngine
+    eng = TraceEngine(write_model(tmp_path / "m", cfg, w), dtype=dtype, max_tokens=max_tokens, block_size=block_size, **kw)
+    m = eng.runner.model
+    for t in m.kv + m.state:                    # a cache row or a state slot that is read before it is written shows as NaN
+        for u in (t or ()):
+            u.fill_(float("nan"))
+    return eng
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def _replay(eng, rid, toks, cuts):
+    """Feed toks in portions ending at `cuts`; returns the logits of every position."""
+    out, lo = [], 0
+    for hi in cuts:
+        out.append(eng.step([{"id": rid, "tokens": toks[lo:hi], "want": list(range(hi - lo))}], [rid] if hi == len(toks) else []))
+        lo = hi
+    return torch.cat(out)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(configs()))
+def test_whole_prompt_and_every_layer_match_the_oracle(tmp_path, name, dtype):
+    cfg, w = make(name)
+    toks = tokens(83, cfg["vocab"], 1)
+    res = []
+    ref = F.forward(cfg, w, toks, res)
+    eng = engine(tmp_path, cfg, w, dtype)
+    eng.runner.model.tap_residuals = []
+    got = eng.step([{"id": "a", "tokens": toks, "want": list(range(len(toks)))}], ["a"])
+    taps = eng.runner.model.tap_residuals
+    assert len(taps) == len(res) == len(cfg["layers"])
+    for i, (a, b) in enumerate(zip(taps, res)):
+        assert close(a, b, dtype), f"layer {i}: {rel_err(a, b)}"
+    assert close(got, ref, dtype), rel_err(got, ref)
+
+
+@pytest.mark.parametrize("name", list(configs()))
+def test_portions_and_token_by_token_decoding_equal_the_whole_prompt(tmp_path, name):
+    cfg, w = make(name, seed=2)
+    n = 70
+    toks = tokens(n, cfg["vocab"], 3)
+    ref = F.forward(cfg, w, toks)
+    eng = engine(tmp_path, cfg, w, "float32", block_size=16)
+    whole = _replay(eng, "w", toks, [n])
+    assert rel_err(whole, ref) < TOL["float32"]
+    schedules = {
+        "token by token from the first": list(range(1, n + 1)),
+        "prompt then decoding": [41] + list(range(42, n + 1)),
+        "portions of two": list(range(2, n + 1, 2)),
+        "portions of changing size, cut at and next to page borders": [15, 16, 17, 32, 35, 47, 48, 50, 64, 65, n],
+        "three then single tokens over a page border": [3] + list(range(4, 20)) + [n],
+    }
+    for what, cuts in schedules.items():
+        got = _replay(eng, what, toks, cuts)
+        assert rel_err(got, ref) < TOL["float32"], what
+        # every row is computed from its own inputs, the cache and the state in a fixed order: no dependence on the cut at all
+        assert torch.equal(got, whole), what
+
+
+def test_window_edges_sinks_far_tokens_and_saved_inputs_show(tmp_path):
+    """The model is sensitive to what the test is about: against an oracle whose window is one key longer or shorter, whose sink is
+    left out, whose slowest decays are a little off or whose convolution misses its oldest tap, the engine is FAR from equal; against
+    the right one it is equal -- in prompts, in portions and in decoding, with windows that end inside a page, at its border and
+    several pages back."""
+    cfg, w = make("all_kinds", seed=5)
+    n = 90
+    toks = tokens(n, cfg["vocab"], 6)
+    ref = F.forward(cfg, w, toks)
+    eng = engine(tmp_path, cfg, w, "float32", block_size=16)
+    got = _replay(eng, "a", toks, [40] + list(range(41, n + 1)))
+    assert rel_err(got, ref) < TOL["float32"]
+    for li, delta in ((0, 1), (0, -1), (3, 1), (3, -1), (4, 1), (4, -1)):
+        other = json.loads(json.dumps(cfg))
+        other["layers"][li]["mixer"]["mask"]["size"] += delta
+        wrong = F.forward(other, w, toks)
+        first = cfg["layers"][li]["mixer"]["mask"]["size"] + min(delta, 0)      # the first position that sees a different key set
+        assert rel_err(got[first:], wrong[first:]) > 100 * TOL["float32"], (li, delta)
+    far = dict(w)
+    far["l0.mix.sink"] = torch.full_like(w["l0.mix.sink"], -60.0)              # as good as no sink
+    assert rel_err(got, F.forward(cfg, far, toks)) > 100 * TOL["float32"]
+    far = dict(w)
+    far["l1.mix.w0"] = torch.where(w["l1.mix.w0"] < -4.0, w["l1.mix.w0"] + 0.5, w["l1.mix.w0"])    # only the slowest channels: far tokens
+    assert rel_err(got[60:], F.forward(cfg, far, toks)[60:]) > 100 * TOL["float32"]
+    far = dict(w)
+    far["l2.mix.A_log"] = torch.where(w["l2.mix.A_log"] < -1.0, w["l2.mix.A_log"] + 0.5, w["l2.mix.A_log"])
+    assert rel_err(got[60:], F.forward(cfg, far, toks)[60:]) > 100 * TOL["float32"]
+    far = dict(w)
+    far["l2.mix.conv"] = w["l2.mix.conv"].clone()
+    far["l2.mix.conv"][:, 0] = 0                                               # the oldest tap: the input three tokens back
+    assert rel_err(got, F.forward(cfg, far, toks)) > 100 * TOL["float32"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(tmp_path, dtype):
+    """Up to three live requests, prompt portions of some beside single tokens of others, in a pool too small for all of them at once:
+    pages and state slots of finished requests (filled by them, never cleared) are taken again."""
+    cfg, w = make("all_kinds", seed=4)
+    V = cfg["vocab"]
+    reqs = {r: tokens(n, V, 40 + i) for i, (r, n) in enumerate([("a", 61), ("b", 7), ("c", 38), ("d", 1), ("e", 50), ("f", 23)])}
+    refs = {r: F.forward(cfg, w, t) for r, t in reqs.items()}
+    eng = engine(tmp_path, cfg, w, dtype, max_tokens=176, block_size=16, max_live=3)
+    at = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    plan = [[("a", 20), ("b", 3)], [("a", 1), ("b", 4), ("c", 2)], [("a", 17), ("c", 1)], [("c", 30), ("a", 1), ("d", 1)],
+            [("a", 22), ("c", 5), ("e", 16)], [("e", 1), ("f", 2)], [("e", 33), ("f", 1)], [("f", 20)]]
+    for step in plan:
+        entries, end = [], []
+        for r, k in step:
+            entries.append({"id": r, "tokens": reqs[r][at[r]:at[r] + k], "want": list(range(k))})
+            at[r] += k
+            if at[r] == len(reqs[r]):
+                end.append(r)
+        out = eng.step(entries, end)
+        lo = 0
+        for r, k in step:
+            got[r].append(out[lo:lo + k])
+            lo += k
+    assert all(at[r] == len(reqs[r]) for r in reqs)
+    assert not eng.live and len(eng.blocks.free_block_ids) == 11 and eng.blocks.free_state_slots == [0, 1, 2]
+    if dtype == "float32":
+        for r in reqs:
+            g = torch.cat(got[r])
+            assert close(g, refs[r], dtype), (r, rel_err(g, refs[r]))
+        for r in ("a", "e"):          # each alone gives exactly the same rows
+            alone = _replay(eng, r + "x", reqs[r], [len(reqs[r])])
+            assert torch.equal(alone, torch.cat(got[r]))
+    else:           # the bf16 bound is a statement about many positions: all requests together
+        assert close(torch.cat([torch.cat(got[r]) for r in reqs]), torch.cat([refs[r] for r in reqs]), dtype)
+
+
+@pytest.mark.parametrize("block_size", [32, 64])
+def test_bf16_fast_forms_through_the_engine_portions_decoding_and_mixed_steps(tmp_path, block_size):
+    """bf16 with 32 / 64-token pages and sizes that the MFMA attention and the register scans take: whole prompt, portions cut at and
+    next to page borders, decoded tokens (the attention's wave-split form), two requests sharing steps; every position against the
+    oracle, the portions against the whole prompt, and the MFMA attention against the scalar form on the same inputs."""
+    cfg, w = make("fast_forms", seed=9)
+    n = 190
+    ta, tb = tokens(n, cfg["vocab"], 30), tokens(77, cfg["vocab"], 31)
+    ra, rb = F.forward(cfg, w, ta), F.forward(cfg, w, tb)
+    eng = engine(tmp_path, cfg, w, "bfloat16", max_tokens=384, block_size=block_size)
+    whole = _replay(eng, "w", ta, [n])
+    assert close(whole, ra, "bfloat16"), rel_err(whole, ra)
+    eng.runner.model.scalar_attention = True
+    scalar = _replay(eng, "s", ta, [n])
+    eng.runner.model.scalar_attention = False
+    assert row_err(whole, scalar.double().cpu()).median() < 0.02
+    cuts = sorted({block_size - 1, block_size, block_size + 1, 2 * block_size + 2, 150} | set(range(151, n + 1)))
+    got = _replay(eng, "c", ta, cuts)
+    assert close(got, ra, "bfloat16"), rel_err(got, ra)
+    assert row_err(got, whole.double().cpu()).median() < 0.02
+    ga, gb, ia, ib = [], [], 0, 0
+    for ka, kb in [(40, 1), (1, 1), (1, 30), (25, 1), (1, 44)] + [(1, 0)] * 10 + [(n - 78, 0)]:
+        entries = []
+        if ka:
+            entries.append({"id": "a", "tokens": ta[ia:ia + ka], "want": list(range(ka))})
+        if kb:
+            entries.append({"id": "b", "tokens": tb[ib:ib + kb], "want": list(range(kb))})
+        ia, ib = ia + ka, ib + kb
+        out = eng.step(entries, [r for r, done in (("a", ia == n), ("b", ib == 77 and kb)) if done])
+        ga.append(out[:ka])
+        gb.append(out[ka:ka + kb])
+    assert ia == n and ib == 77
+    assert close(torch.cat(ga), ra, "bfloat16") and close(torch.cat(gb), rb, "bfloat16")
+
+
+def test_fast_forms_in_fp32_rows_equal_for_any_cut(tmp_path):
+    """The register scans also run in the fp32 element mode; their rows do not depend on the cut either."""
+    cfg, w = make("fast_forms", seed=10)
+    n = 100
+    toks = tokens(n, cfg["vocab"], 12)
+    ref = F.forward(cfg, w, toks)
+    eng = engine(tmp_path, cfg, w, "float32", max_tokens=256, block_size=32)
+    whole = _replay(eng, "w", toks, [n])
+    assert rel_err(whole, ref) < TOL["float32"]
+    got = _replay(eng, "c", toks, [7, 8, 9, 17, 31, 32, 33, 60] + list(range(61, n + 1)))
+    assert torch.equal(got, whole)
+
+
+def test_long_decoding_over_many_pages(tmp_path):
+    cfg, w = make("all_kinds", seed=8)
+    n = 230
+    toks = tokens(n, cfg["vocab"], 9)
+    ref = F.forward(cfg, w, toks)
+    eng = engine(tmp_path, cfg, w, "float32", max_tokens=256, block_size=16)
+    got = _replay(eng, "a", toks, [5] + list(range(6, n + 1)))
+    assert rel_err(got, ref) < TOL["float32"]
+    eng16 = engine(tmp_path, cfg, w, "bfloat16", max_tokens=256, block_size=16)
+    got16 = _replay(eng16, "a", toks, [5] + list(range(6, n + 1)))
+    assert close(got16, ref, "bfloat16"), rel_err(got16, ref)
+
+
+def test_pool_and_live_limits_are_enforced(tmp_path):
+    cfg, w = make("ones")
+    eng = engine(tmp_path, cfg, w, "float32", max_tokens=64, block_size=16, max_live=2)
+    eng.step([{"id": "a", "tokens": [1] * 20, "want": []}, {"id": "b", "tokens": [2] * 20, "want": []}])
+    with pytest.raises(RuntimeError):
+        eng.step([{"id": "c", "tokens": [3], "want": []}])
+    eng.step([], ["a"])
+    eng.step([{"id": "c", "tokens": [3] * 30, "want": [29]}])
+    with pytest.raises(RuntimeError):
+        eng.step([{"id": "b", "tokens": [2] * 20, "want": []}])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_llm_generate(tmp_path, dtype):
+    """The framework's own entry point and scheduler: batched prefill, batched decode (hipGraph replays), pages and state slots from the
+    scheduler's block manager (three slots for four prompts), argmax kernels."""
+    from ssd_amd import LLM, SamplingParams
+    cfg, w = make("all_kinds", seed=7)
+    path = write_model(tmp_path / "m", cfg, w)
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (5, 19, 1, 34)]
+    new = 24
+    llm = LLM(path, dtype=dtype, kvcache_block_size=16, num_kvcache_blocks=32, max_num_seqs=3, max_model_len=128,
+              max_num_batched_tokens=128)
+    outs, _ = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new, ignore_eos=True), use_tqdm=False)
+    assert len(outs) == len(prompts)
+    del llm
+    eng = engine(tmp_path / "t", cfg, w, dtype, max_tokens=256)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        gen = o["token_ids"]
+        assert len(gen) == new
+        # teacher forcing: every generated token is the argmax of its step.  The argmax kernels read the logits rounded to bf16, so a
+        # runner-up within that rounding of the top may win.  Against the oracle in fp32; in bf16 (where a router decision flipped by
+        # rounding moves these tiny models' logits a lot) against the same arithmetic fed step by step through the trace engine.
+        seq = p + gen[:-1]
+        if dtype == "float32":
+            lg = F.forward(cfg, w, seq)[len(p) - 1:]
+        else:
+            lg = eng.step([{"id": str(i), "tokens": seq, "want": list(range(len(p) - 1, len(seq)))}], [str(i)]).double().cpu()
+        top = lg.max(-1).values
+        chosen = lg[torch.arange(new), torch.tensor(gen)]
+        assert ((top - chosen) <= 2.0 ** -7 * top.abs() + 1e-3 * lg.std()).all(), (i, (top - chosen).max())
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_configurations_in_both_modes_whole_and_in_portions(tmp_path, seed):
+    g = torch.Generator().manual_seed(100 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    layers = []
+    for i in range(r(2, 5)):
+        kind = r(0, 2)
+        mlp = [None, F.dense_mlp(8 * r(1, 6)), None][kind] if kind < 2 else None
+        if kind == 2:
+            E = r(1, 7)
+            mlp = F.moe_mlp(experts=E, top=r(1, E), ff=8 * r(1, 4), limit=0.5 + 0.5 * r(0, 3))
+        mix = r(0, 2)
+        if mix == 0:
+            G = r(1, 3)
+            layers.append(F.attention_layer(heads=G * r(1, 4), kv_heads=G, dim=r(1, 5) * 8, vdim=r(1, 40), scale=0.2 * r(1, 5),
+                                            softcap=[0, 5.0, 20.0][r(0, 2)], window=r(0, 40), mlp=mlp))
+        elif mix == 1:
+            layers.append(F.wkv_layer(heads=r(1, 4), dim=r(1, 5) * 8, decay_rank=r(1, 9), mlp=mlp))
+        else:
+            G = r(1, 3)
+            H = G * r(1, 3)
+            vd = r(1, 5) * 4
+            ng = [d for d in (1, 2, 4, H) if (H * vd) % d == 0][r(0, 2) % 3]
+            layers.append(F.mamba2_layer(heads=H, vdim=vd, state=r(1, 5) * 4, groups=G, conv=r(1, 5), norm_groups=ng, mlp=mlp))
+        if i and r(0, 3) == 0:          # borrow the weights of an earlier layer of its own
+            src = r(0, i - 1)
+            if "weights_of" not in layers[src]:
+                layers[i] = json.loads(json.dumps(layers[src]))
+                layers[i]["weights_of"] = src
+    cfg = F.make_config(layers, vocab=r(20, 150), width=8 * r(3, 12), logit_scale=0.5 * r(1, 4), logit_softcap=[0, 10.0, 30.0][r(0, 2)])
+    w = F.random_model(cfg, seed)
+    toks = tokens(60, cfg["vocab"], seed)
+    ref = F.forward(cfg, w, toks)
+    for dtype in ("float32", "bfloat16"):
+        eng = engine(tmp_path / dtype, cfg, w, dtype, max_tokens=128, block_size=16)
+        whole = _replay(eng, "w", toks, [60])
+        assert close(whole, ref, dtype), (dtype, rel_err(whole, ref))
+        parts = _replay(eng, "p", toks, [7, 9, 31, 32, 33] + list(range(34, 61)))
+        assert close(parts, ref, dtype), (dtype, rel_err(parts, ref))
