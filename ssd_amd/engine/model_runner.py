@@ -113,9 +113,10 @@ class ModelRunner:
                 t = torch.tensor([num_kvcache_blocks], dtype=torch.int64, device=device)
                 dist.all_reduce(t, op=dist.ReduceOp.MIN, group=tp_group)
                 num_kvcache_blocks = int(t.item())
-        if getattr(self.model, "state_slots", 0):
-            # a recurrent model reuses no prefix pages: max_num_seqs sequences of max_model_len tokens are all it can ever hold
-            num_kvcache_blocks = min(num_kvcache_blocks, self.max_bs * self.max_blocks + 1)
+            if getattr(self.model, "state_slots", 0):
+                # a recurrent model reuses no prefix pages: max_num_seqs sequences of max_model_len tokens are all it can ever hold.
+                # Only a count sized from free memory is cut: a count the caller gave is the number of ids its block manager hands out
+                num_kvcache_blocks = min(num_kvcache_blocks, self.max_bs * self.max_blocks + 1)
         assert num_kvcache_blocks > 0, "KV cache does not fit"
         self.num_kvcache_blocks = num_kvcache_blocks
         self.model.alloc_kv(num_kvcache_blocks)

@@ -35,6 +35,7 @@ class TraceEngine:
                                       num_kvcache_blocks=pool)
         else:
             self.runner = runner_factory(self.config)
+        assert getattr(self.runner, "num_kvcache_blocks", pool) == pool, "the runner's cache must hold every page the block manager hands out"
         # a model with recurrent layers: max_live state slots, taken and returned with a request's pages
         recurrent = bool(getattr(self.config.hf_config, "recurrent", False))
         self.blocks = BlockManager(pool, block_size, max_model_len=cap, prefix_cache=False, state_slots=max_live if recurrent else 0)

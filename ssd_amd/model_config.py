@@ -461,7 +461,7 @@ class FomunexConfig:
     def complete_from_checkpoint(self, model_dir: str) -> None:
         """Sizes that only a tensor's shape gives (the decay rank of time-mixing layers): read from the safetensors headers."""
         need = [i for i, l in enumerate(self.layers) if l.mixer.kind == "wkv" and not l.mixer.decay_rank]
-        if not need:
+        if not need and self.max_position_embeddings > 0:
             return
         import glob
         import struct
@@ -475,6 +475,10 @@ class FomunexConfig:
             if name not in shapes:
                 raise ValueError(f"Fomunex: {name} not found under {model_dir}")
             self.layers[i].mixer.decay_rank = int(shapes[name][0])
+        if self.max_position_embeddings <= 0:          # config.json without max_positions: the position table's rows
+            if "pos" not in shapes:
+                raise ValueError(f"Fomunex: neither max_positions nor a position table under {model_dir}")
+            self.max_position_embeddings = int(shapes["pos"][0])
 
     @staticmethod
     def from_json(cfg: dict) -> "FomunexConfig":
@@ -483,7 +487,8 @@ class FomunexConfig:
             m, kind = lc["mixer"], lc["type"]
             if kind == "attention":
                 mask = m.get("mask") or {}
-                mixer = WindowAttention(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]),
+                mixer = WindowAttention(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]),
+                                        float(m["scale"]) if m.get("scale") is not None else int(m["dim"]) ** -0.5,
                                         float(m.get("softcap") or 0.0), int(mask.get("size") or 0))
                 if mixer.heads % mixer.kv_heads:
                     raise ValueError("Fomunex: heads must be a multiple of kv_heads")
@@ -503,7 +508,7 @@ class FomunexConfig:
                     mlp = PolyNormMLP(int(ml["ff"]))
                 elif ml["kind"] == "moe":
                     mlp = SigmoidRoutedMLP(int(ml["router"]["experts"]), int(ml["router"]["top"]), int(ml["expert"]["ff"]),
-                                           float(ml["expert"]["limit"]))
+                                           float(ml["expert"].get("limit") or 3.0e38))
                     if not 1 <= mlp.top <= mlp.experts:
                         raise ValueError("Fomunex: top does not fit the experts")
                 else:
@@ -515,8 +520,8 @@ class FomunexConfig:
         for l in layers:        # a layer that borrows weights has its source's sizes, also the one a tensor's shape gives
             if l.mixer.kind == "wkv" and not l.mixer.decay_rank:
                 l.mixer.decay_rank = layers[l.weights_of].mixer.decay_rank
-        return FomunexConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, int(cfg["max_positions"]),
-                             float(cfg.get("logit_scale", 1.0)), float(cfg.get("logit_softcap") or 0.0))
+        return FomunexConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, int(cfg.get("max_positions") or 0),
+                             float(cfg.get("logit_scale") or 1.0), float(cfg.get("logit_softcap") or 0.0))
 
 
 # config.json "architecture" values that are read by this package's own readers (everything else goes through transformers' AutoConfig)

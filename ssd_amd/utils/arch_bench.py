@@ -7,7 +7,13 @@ key / value / output projection sizes (two 64-wide maps per head = one 128-wide 
 --workload zerusun: the Zerusun decoder (layers alternate latent attention with a sliding window and linear attention over a recurrent
 state; routed three-matrix experts with group-limited choice and a gated shared expert; the stack is one loop of one pass) beside
 the closest existing family, Fatulix, at equal size: the same width, layers, vocabulary, experts, top and feed-forward parameters per
-token (three-matrix experts of 2/3 the two-matrix experts' ff), mixers of about the same parameter count."""
+token (three-matrix experts of 2/3 the two-matrix experts' ff), mixers of about the same parameter count.
+
+--workload fomunex: the Fomunex decoder (pre-norm layers; windowed attention with a sink / time mixing / windowed attention / state
+space; sigmoid-routed clamped-GLU experts and one PolyNorm dense feed-forward) beside the closest existing family, Zerusun (fp32
+residual, a windowed attention over a paged cache next to a recurrent mixer over state slots, routed three-matrix experts), at equal
+size: the same width, layers, vocabulary, experts, top and active feed-forward parameters per token, the same window, mixers of about
+the same parameter count."""
 from __future__ import annotations
 
 import json
@@ -18,8 +24,9 @@ import torch
 from ssd_amd.config import Config
 from ssd_amd.engine.block_manager import BlockManager
 from ssd_amd.engine.sequence import Sequence
-from ssd_amd.model_config import (DiffAttention, FatulixConfig, FatulixLayer, GroupRoutedMLP, LatentAttention, LightningAttention, ModelConfig,
-                                  RopeSpec, RoutedMLP, ZerusunConfig, ZerusunLayer)
+from ssd_amd.model_config import (DiffAttention, FatulixConfig, FatulixLayer, FomunexConfig, FomunexLayer, GroupRoutedMLP, LatentAttention,
+                                  LightningAttention, Mamba2Mixer, ModelConfig, PolyNormMLP, RopeSpec, RoutedMLP, SigmoidRoutedMLP,
+                                  WindowAttention, WkvMixer, ZerusunConfig, ZerusunLayer)
 
 VOCAB = 32000
 SIZES = {
@@ -50,6 +57,22 @@ def zerusun_models(size: str):
     return zer, fat
 
 
+def fomunex_models(size: str):
+    """(Fomunex, Zerusun) of equal size: the experts carry what Zerusun's experts and its shared expert carry per token together."""
+    W, L, Hh, G, E, top, ff, sff, inter = SIZES[size]
+    zer, _ = zerusun_models(size)
+    ffx = (ff + sff // top) * 2 // 3
+    moe = SigmoidRoutedMLP(E, top, ffx, 7.0)
+    dense = PolyNormMLP(3 * top * ffx // 2)                  # two matrices instead of top * three
+    att = WindowAttention(Hh, G, 128, 128, 0.125, 30.0, 1024)
+    layers = [FomunexLayer(att, moe, 0), FomunexLayer(WkvMixer(W // 128, 64, 64), dense, 1), FomunexLayer(att, moe, 2),
+              FomunexLayer(Mamba2Mixer(W // 64, 64, 128, 1, 4, 1), moe, 3)]
+    fom = FomunexConfig(VOCAB, W, 1e-5, (layers * (L // 4 + 1))[:L], 8192, 1.0, 30.0)
+    for i, l in enumerate(fom.layers):
+        fom.layers[i] = FomunexLayer(l.mixer, l.mlp, i)
+    return fom, zer
+
+
 def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
     from ssd_amd.engine.model_runner import ModelRunner
     bs = 256
@@ -58,6 +81,7 @@ def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
                     max_num_batched_tokens=max(max_len, 4096), num_kvcache_blocks=blocks)
     Sequence.block_size = bs
     runner = ModelRunner(config, cfg, is_draft=False, device=torch.device("cuda", 0), weights_seed=0, num_kvcache_blocks=blocks)
+    assert runner.num_kvcache_blocks == blocks, "the runner's cache must hold every page the block manager hands out"
     return runner, BlockManager(blocks, bs, max_model_len=max_len, prefix_cache=False,
                                 state_slots=batch if getattr(cfg, "recurrent", False) else 0)
 
@@ -146,6 +170,35 @@ def run_zerusun(args) -> dict:
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights, random tokens)",
             "config": {"model": "zerusun-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
             "closest_model_value": results[k]["fatulix_equal_size"]["decode_tok_s"], "sizes": results}
+
+
+def run_fomunex(args) -> dict:
+    steps, warmup = args.steps, args.warmup
+    prompt_len = args.input_len if args.input_len != 128 else 2048
+    results = {}
+    sizes = list(SIZES) if getattr(args, "arch_size", "all") == "all" else [args.arch_size]
+    batches = (1, 8) if not getattr(args, "arch_batch", 0) else (args.arch_batch,)
+    only = getattr(args, "arch_only", "both")
+    for size in sizes:
+        fom, zer = fomunex_models(size)
+        for batch in batches:
+            key = f"{size} prompt={prompt_len} batch={batch}"
+            results[key] = {}
+            if only in ("both", "fomunex"):
+                results[key]["fomunex"] = measure(fom, prompt_len, batch, steps, warmup)
+            if only in ("both", "zerusun"):
+                results[key]["zerusun_equal_size"] = measure(zer, prompt_len, batch, steps, warmup)
+            print(f"[arch_bench] {key}: {json.dumps(results[key])}", flush=True)
+    k = f"w4096 prompt={prompt_len} batch=8"
+    if k not in results or len(results[k]) < 2:
+        return {"metric": "Fomunex / equal-size Zerusun throughput (partial run)", "sizes": results}
+    return {"metric": "decode tokens/s, Fomunex w4096 (4 layers: windowed attention / time mixing / windowed attention / state space, 16 "
+                      "experts top 2), batch 8, beside an equal-size Zerusun decoder",
+            "value": results[k]["fomunex"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": results[k]["fomunex"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights, random tokens)",
+            "config": {"model": "fomunex-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
+            "closest_model_value": results[k]["zerusun_equal_size"]["decode_tok_s"], "sizes": results}
 
 
 def run(args) -> dict:

@@ -35,14 +35,24 @@ def rel_err(got, ref) -> float:
     return float(row_err(got, ref).max())
 
 
-def close(got, ref, dtype) -> bool:
-    """fp32: every position within 1e-4 of the spread.  bf16: rounding of GEMM inputs, and now and then a router decision made the other
+def oracle(cfg, w, toks):
+    """(logits, per-position rounding floor).  Some positions amplify rounding by orders of magnitude -- at a sequence's first token the
+    time-mixing output is ONE number times the value vector, divided by its own root mean square: when that number is near zero the
+    norm's eps decides, and 1e-7 of rounding comes out as 1e-4.  The floor is what fp32 rounding of every sublayer's input alone does
+    to the float64 statement; a position's bound is the larger of the fixed one and 50 floors."""
+    ref = F.forward(cfg, w, toks)
+    low = F.forward(cfg, w, toks, round_input=lambda t: t.float().double())
+    return ref, row_err(low, ref)
+
+
+def close(got, ref, dtype, floor=None) -> bool:
+    """fp32: every position within 1e-4 of the spread (or 50 rounding floors, see oracle()).  bf16: rounding of GEMM inputs, and now and then a router decision made the other
     way at a near-tie, which in these tiny models (a few experts, a few values wide) moves that position by tens of percent: the median
     within 5 %, nine positions in ten within 20 %, all finite.  What a schedule, the cache or the state could get wrong is pinned by
     the fp32 runs."""
     e = row_err(got, ref)
     if dtype == "float32":
-        return bool(e.max() < TOL[dtype])
+        return bool((e < (TOL[dtype] if floor is None else torch.clamp(50 * floor, min=TOL[dtype]))).all())
     return bool(torch.isfinite(got).all() and e.median() < 0.05 and e.quantile(0.9) < 0.2)
 
 
@@ -109,14 +119,15 @@ def test_whole_prompt_and_every_layer_match_the_oracle(tmp_path, name, dtype):
     toks = tokens(83, cfg["vocab"], 1)
     res = []
     ref = F.forward(cfg, w, toks, res)
+    floor = oracle(cfg, w, toks)[1]
     eng = engine(tmp_path, cfg, w, dtype)
     eng.runner.model.tap_residuals = []
     got = eng.step([{"id": "a", "tokens": toks, "want": list(range(len(toks)))}], ["a"])
     taps = eng.runner.model.tap_residuals
     assert len(taps) == len(res) == len(cfg["layers"])
     for i, (a, b) in enumerate(zip(taps, res)):
-        assert close(a, b, dtype), f"layer {i}: {rel_err(a, b)}"
-    assert close(got, ref, dtype), rel_err(got, ref)
+        assert close(a, b, dtype, floor), f"layer {i}: {rel_err(a, b)}"
+    assert close(got, ref, dtype, floor), rel_err(got, ref)
 
 
 @pytest.mark.parametrize("name", list(configs()))
@@ -124,10 +135,10 @@ def test_portions_and_token_by_token_decoding_equal_the_whole_prompt(tmp_path, n
     cfg, w = make(name, seed=2)
     n = 70
     toks = tokens(n, cfg["vocab"], 3)
-    ref = F.forward(cfg, w, toks)
+    ref, floor = oracle(cfg, w, toks)
     eng = engine(tmp_path, cfg, w, "float32", block_size=16)
     whole = _replay(eng, "w", toks, [n])
-    assert rel_err(whole, ref) < TOL["float32"]
+    assert close(whole, ref, "float32", floor), rel_err(whole, ref)
     schedules = {
         "token by token from the first": list(range(1, n + 1)),
         "prompt then decoding": [41] + list(range(42, n + 1)),
@@ -137,7 +148,6 @@ def test_portions_and_token_by_token_decoding_equal_the_whole_prompt(tmp_path, n
     }
     for what, cuts in schedules.items():
         got = _replay(eng, what, toks, cuts)
-        assert rel_err(got, ref) < TOL["float32"], what
         # every row is computed from its own inputs, the cache and the state in a fixed order: no dependence on the cut at all
         assert torch.equal(got, whole), what
 
@@ -150,10 +160,10 @@ def test_window_edges_sinks_far_tokens_and_saved_inputs_show(tmp_path):
     cfg, w = make("all_kinds", seed=5)
     n = 90
     toks = tokens(n, cfg["vocab"], 6)
-    ref = F.forward(cfg, w, toks)
+    ref, floor = oracle(cfg, w, toks)
     eng = engine(tmp_path, cfg, w, "float32", block_size=16)
     got = _replay(eng, "a", toks, [40] + list(range(41, n + 1)))
-    assert rel_err(got, ref) < TOL["float32"]
+    assert close(got, ref, "float32", floor), rel_err(got, ref)
     for li, delta in ((0, 1), (0, -1), (3, 1), (3, -1), (4, 1), (4, -1)):
         other = json.loads(json.dumps(cfg))
         other["layers"][li]["mixer"]["mask"]["size"] += delta
@@ -182,7 +192,8 @@ def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(tmp_p
     cfg, w = make("all_kinds", seed=4)
     V = cfg["vocab"]
     reqs = {r: tokens(n, V, 40 + i) for i, (r, n) in enumerate([("a", 61), ("b", 7), ("c", 38), ("d", 1), ("e", 50), ("f", 23)])}
-    refs = {r: F.forward(cfg, w, t) for r, t in reqs.items()}
+    both = {r: oracle(cfg, w, t) for r, t in reqs.items()}
+    refs = {r: v[0] for r, v in both.items()}
     eng = engine(tmp_path, cfg, w, dtype, max_tokens=176, block_size=16, max_live=3)
     at = {r: 0 for r in reqs}
     got = {r: [] for r in reqs}
@@ -205,7 +216,7 @@ def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(tmp_p
     if dtype == "float32":
         for r in reqs:
             g = torch.cat(got[r])
-            assert close(g, refs[r], dtype), (r, rel_err(g, refs[r]))
+            assert close(g, refs[r], dtype, both[r][1]), (r, rel_err(g, refs[r]))
         for r in ("a", "e"):          # each alone gives exactly the same rows
             alone = _replay(eng, r + "x", reqs[r], [len(reqs[r])])
             assert torch.equal(alone, torch.cat(got[r]))
@@ -253,10 +264,10 @@ def test_fast_forms_in_fp32_rows_equal_for_any_cut(tmp_path):
     cfg, w = make("fast_forms", seed=10)
     n = 100
     toks = tokens(n, cfg["vocab"], 12)
-    ref = F.forward(cfg, w, toks)
+    ref, floor = oracle(cfg, w, toks)
     eng = engine(tmp_path, cfg, w, "float32", max_tokens=256, block_size=32)
     whole = _replay(eng, "w", toks, [n])
-    assert rel_err(whole, ref) < TOL["float32"]
+    assert close(whole, ref, "float32", floor), rel_err(whole, ref)
     got = _replay(eng, "c", toks, [7, 8, 9, 17, 31, 32, 33, 60] + list(range(61, n + 1)))
     assert torch.equal(got, whole)
 
@@ -265,10 +276,10 @@ def test_long_decoding_over_many_pages(tmp_path):
     cfg, w = make("all_kinds", seed=8)
     n = 230
     toks = tokens(n, cfg["vocab"], 9)
-    ref = F.forward(cfg, w, toks)
+    ref, floor = oracle(cfg, w, toks)
     eng = engine(tmp_path, cfg, w, "float32", max_tokens=256, block_size=16)
     got = _replay(eng, "a", toks, [5] + list(range(6, n + 1)))
-    assert rel_err(got, ref) < TOL["float32"]
+    assert close(got, ref, "float32", floor), rel_err(got, ref)
     eng16 = engine(tmp_path, cfg, w, "bfloat16", max_tokens=256, block_size=16)
     got16 = _replay(eng16, "a", toks, [5] + list(range(6, n + 1)))
     assert close(got16, ref, "bfloat16"), rel_err(got16, ref)
@@ -349,10 +360,10 @@ def test_random_configurations_in_both_modes_whole_and_in_portions(tmp_path, see
     cfg = F.make_config(layers, vocab=r(20, 150), width=8 * r(3, 12), logit_scale=0.5 * r(1, 4), logit_softcap=[0, 10.0, 30.0][r(0, 2)])
     w = F.random_model(cfg, seed)
     toks = tokens(60, cfg["vocab"], seed)
-    ref = F.forward(cfg, w, toks)
+    ref, floor = oracle(cfg, w, toks)
     for dtype in ("float32", "bfloat16"):
         eng = engine(tmp_path / dtype, cfg, w, dtype, max_tokens=128, block_size=16)
         whole = _replay(eng, "w", toks, [60])
-        assert close(whole, ref, dtype), (dtype, rel_err(whole, ref))
+        assert close(whole, ref, dtype, floor), (dtype, rel_err(whole, ref))
         parts = _replay(eng, "p", toks, [7, 9, 31, 32, 33] + list(range(34, 61)))
-        assert close(parts, ref, dtype), (dtype, rel_err(parts, ref))
+        assert close(parts, ref, dtype, floor), (dtype, rel_err(parts, ref))
