@@ -47,7 +47,7 @@ token_shift_mix_kernel(const T* __restrict__ hn, const T* __restrict__ mu, const
   const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
   const bool from_batch = t > row0, zero = !from_batch && positions[t] == 0;
   const float* st = shift_state + (size_t)state_slots[b] * W;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += 256 * gridDim.y) {
     const float h = ldf<T>(hn + (size_t)t * W + c);
     const float prev = from_batch ? ldf<T>(hn + (size_t)(t - 1) * W + c) : (zero ? 0.f : st[c]);
     for (int s = 0; s < S; ++s) stf<T>(out + ((size_t)t * S + s) * W + c, fmaf(prev - h, ldf<T>(mu + (size_t)s * W + c), h));
@@ -123,8 +123,10 @@ wkv_scan_kernel(const float* __restrict__ proj, long ld, int r_off, int k_off, i
   }
   __syncthreads();
   for (int i = tid; i < D * D; i += 256) sp[i] = S[i];
-  if (h == 0)          // the last row of the portion is the next portion's "previous token"
-    for (int c = tid; c < W; c += 256) shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
+  // the last row of the portion is the next portion's "previous token": every head's workgroup saves its share of the columns
+  const int chunk = (W + H - 1) / H;
+  for (int c = h * chunk + tid; c < min(W, (h + 1) * chunk); c += 256)
+    shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
 }
 
 template <typename T>
@@ -156,11 +158,12 @@ causal_conv_silu_kernel(const float* __restrict__ proj, long ld, int col_off, in
 
 constexpr int CONV_MAX_TAPS = 16;
 
+// Channels [c_begin, c_end) of the slot's saved convolution inputs: saved row i holds the input of position p0 + n - (taps - 1) + i.
 __device__ __forceinline__ void save_conv_state(const float* proj, long ld, int conv_off, int C, float* conv_state, int taps, int slot,
-                                                int row0, int row1, long p0) {
+                                                int row0, int row1, long p0, int c_begin, int c_end) {
   const int n = row1 - row0, K1 = taps - 1;
   float* st = conv_state + (size_t)slot * K1 * C;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  for (int c = c_begin + threadIdx.x; c < c_end; c += 256) {
     float keep[CONV_MAX_TAPS];
 #pragma unroll
     for (int i = 0; i < CONV_MAX_TAPS; ++i) {
@@ -218,8 +221,10 @@ ssd_scan_kernel(const float* __restrict__ xbc, long ldx, int x_off, int b_off, i
   }
   __syncthreads();
   for (int i = tid; i < N * Dv; i += 256) sp[i] = S[i];
-  if (h == 0 && taps > 1)      // the slot's last taps - 1 convolution inputs: saved row i holds the input of position p0 + n - (taps - 1) + i
-    save_conv_state(proj, ld, conv_off, C, conv_state, taps, slot, row0, row1, p0);
+  if (taps > 1) {              // the slot's last taps - 1 convolution inputs: every head's workgroup saves its share of the channels
+    const int chunk = (C + H - 1) / H;
+    save_conv_state(proj, ld, conv_off, C, conv_state, taps, slot, row0, row1, p0, h * chunk, min(C, (h + 1) * chunk));
+  }
 }
 
 // Register form of both scans (state rows D = 8 * EPT with EPT in {4, 8, 16, 32}, Dv % 32 == 0): a workgroup owns 32 state columns of one
@@ -243,7 +248,6 @@ scan_reg_kernel(WkvArgs wa, SsdArgs sa, const int64_t* __restrict__ positions, c
   constexpr int TB = 8, NG = 8, CB = 32, D = NG * EPT;
   __shared__ float sq[TB][D], sk[TB][D], sd[TB][MODE == 0 ? D : 1];
   __shared__ float sv[TB][CB];
-  __shared__ float sdt[TB];
   __shared__ float po[TB][NG][CB];
   const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CB, tid = threadIdx.x;
   const int g = tid >> 5, e = tid & 31;
@@ -262,34 +266,57 @@ scan_reg_kernel(WkvArgs wa, SsdArgs sa, const int64_t* __restrict__ positions, c
   }
   const int grp = MODE == 1 ? h / (H / sa.G) : 0;
   const float a = MODE == 1 ? -expf(sa.a_log[h]) : 0.f, dtb = MODE == 1 ? sa.dt_bias[h] : 0.f, skip = MODE == 1 ? sa.skip[h] : 0.f;
+  // raw values of the next batch travel in registers while the current batch is computed (a batch is short: without this every
+  // batch would wait a full memory round trip)
+  constexpr int QK = TB * D / 256;         // q / k / decay elements of a batch per thread
+  float rq[QK], rk[QK], rw[QK], w0r[QK], rv = 0.f;
+#pragma unroll
+  for (int c = 0; c < QK; ++c) w0r[c] = MODE == 0 ? wa.w0[h * D + (tid + 256 * c) % D] : 0.f;
+  auto fetch = [&](int r) {
+    const int nb = row1 - r < TB ? row1 - r : TB;
+#pragma unroll
+    for (int c = 0; c < QK; ++c) {
+      const int idx = tid + 256 * c, tt = idx / D, d = idx % D;
+      rq[c] = rk[c] = rw[c] = 0.f;
+      if (tt < nb) {
+        if (MODE == 0) {
+          const float* pr = wa.proj + (size_t)(r + tt) * wa.ld + h * D + d;
+          rq[c] = pr[wa.r_off];
+          rk[c] = pr[wa.k_off];
+          rw[c] = wa.ww[(size_t)(r + tt) * wa.ldw + h * D + d];
+        } else {
+          const float* xr = sa.xbc + (size_t)(r + tt) * sa.ldx + grp * D + d;
+          rq[c] = xr[sa.c_off];
+          rk[c] = xr[sa.b_off];
+          rw[c] = sa.proj[(size_t)(r + tt) * sa.ld + sa.dt_off + h];          // the row's raw step size
+        }
+      }
+    }
+    rv = 0.f;
+    if (g < nb)
+      rv = MODE == 0 ? wa.proj[(size_t)(r + g) * wa.ld + wa.v_off + h * Dv + c0 + e]
+                     : sa.xbc[(size_t)(r + g) * sa.ldx + sa.x_off + h * Dv + c0 + e];
+  };
+  fetch(row0);
   for (int r = row0; r < row1; r += TB) {
     const int nb = row1 - r < TB ? row1 - r : TB;
     __syncthreads();                      // the previous batch's readers are done
-    if (MODE == 1) {
-      if (tid < nb) {
-        const float dt = softplusf_(sa.proj[(size_t)(r + tid) * sa.ld + sa.dt_off + h] + dtb);
-        sdt[tid] = dt;
-        sd[tid][0] = expf(a * dt);
-      }
-      __syncthreads();
-    }
-    for (int idx = tid; idx < nb * D; idx += 256) {
-      const int tt = idx / D, d = idx % D;
+#pragma unroll
+    for (int c = 0; c < QK; ++c) {
+      const int idx = tid + 256 * c, tt = idx / D, d = idx % D;
+      sq[tt][d] = rq[c];
       if (MODE == 0) {
-        const float* pr = wa.proj + (size_t)(r + tt) * wa.ld + h * D + d;
-        sq[tt][d] = pr[wa.r_off];
-        sk[tt][d] = pr[wa.k_off];
-        sd[tt][d] = expf(-expf(wa.ww[(size_t)(r + tt) * wa.ldw + h * D + d] + wa.w0[h * D + d]));
+        sk[tt][d] = rk[c];
+        sd[tt][d] = expf(-expf(rw[c] + w0r[c]));
       } else {
-        const float* xr = sa.xbc + (size_t)(r + tt) * sa.ldx + grp * D + d;
-        sq[tt][d] = xr[sa.c_off];
-        sk[tt][d] = sdt[tt] * xr[sa.b_off];
+        const float dt = softplusf_(rw[c] + dtb);
+        sk[tt][d] = dt * rk[c];
+        if (d == 0) sd[tt][0] = expf(a * dt);
       }
     }
-    if (g < nb)
-      sv[g][e] = MODE == 0 ? wa.proj[(size_t)(r + g) * wa.ld + wa.v_off + h * Dv + c0 + e]
-                           : sa.xbc[(size_t)(r + g) * sa.ldx + sa.x_off + h * Dv + c0 + e];
+    sv[g][e] = rv;
     __syncthreads();
+    if (r + TB < row1) fetch(r + TB);
     for (int tt = 0; tt < nb; ++tt) {
       const float ve = sv[tt][e];
       float o = 0.f;
@@ -318,12 +345,15 @@ scan_reg_kernel(WkvArgs wa, SsdArgs sa, const int64_t* __restrict__ positions, c
   }
 #pragma unroll
   for (int n = 0; n < EPT; ++n) sp[(size_t)(g + NG * n) * Dv] = S[n];
-  if (h == 0 && blockIdx.z == 0) {
-    if (MODE == 0) {
-      for (int c = tid; c < W; c += 256) shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
-    } else if (sa.taps > 1) {
-      save_conv_state(sa.proj, sa.ld, sa.conv_off, sa.C, sa.conv_state, sa.taps, slot, row0, row1, p0);
-    }
+  // the slot's saved rows (token shift / convolution inputs): every workgroup of the sequence saves its share of the columns
+  const int wg = h * gridDim.z + blockIdx.z, nwg = H * gridDim.z;
+  if (MODE == 0) {
+    const int chunk = (W + nwg - 1) / nwg;
+    for (int c = wg * chunk + tid; c < min(W, (wg + 1) * chunk); c += 256)
+      shift_state[(size_t)slot * W + c] = ldf<T>(hn + (size_t)(row1 - 1) * W + c);
+  } else if (sa.taps > 1) {
+    const int chunk = (sa.C + nwg - 1) / nwg;
+    save_conv_state(sa.proj, sa.ld, sa.conv_off, sa.C, sa.conv_state, sa.taps, slot, row0, row1, p0, wg * chunk, min(sa.C, (wg + 1) * chunk));
   }
 }
 
@@ -366,11 +396,13 @@ extern "C" int ssd_token_shift_mix(const void* hn_rows, const void* mu, const fl
                                    int S, int f32, void* stream) {
   if (!hn_rows || !mu || !shift_state || !positions || !state_slots || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || W <= 0 || S <= 0 || B <= 0 || (!cu_q && q_per_seq <= 0)) return SSD_ERR_SHAPE;
+  const int cbk = (W + 255) / 256;
+  const dim3 grid(T, T >= 256 ? 1 : (cbk < 32 ? cbk : 32));          // few rows: a row's columns spread over workgroups
   if (f32)
-    hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)hn_rows, (const float*)mu,
+    hipLaunchKernelGGL(token_shift_mix_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)hn_rows, (const float*)mu,
                        shift_state, positions, cu_q, q_per_seq, state_slots, B, (float*)out_rows, W, S);
   else
-    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)hn_rows,
+    hipLaunchKernelGGL(token_shift_mix_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)hn_rows,
                        (const bf16_t*)mu, shift_state, positions, cu_q, q_per_seq, state_slots, B, (bf16_t*)out_rows, W, S);
   return LAUNCH_OK();
 }
