@@ -178,7 +178,7 @@ def dense_mlp(ff: int = 40) -> dict:
     return {"kind": "dense", "ff": ff}
 
 
-def moe_mlp(experts: int = 5, top: int = 2, ff: int = 24, limit: float = 1.5) -> dict:
+def moe_mlp(experts: int = 5, top: int = 2, ff: int = 24, limit: float = 1.25) -> dict:
     return {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
 
 

@@ -367,3 +367,31 @@ def test_random_configurations_in_both_modes_whole_and_in_portions(tmp_path, see
         assert close(whole, ref, dtype, floor), (dtype, rel_err(whole, ref))
         parts = _replay(eng, "p", toks, [7, 9, 31, 32, 33] + list(range(34, 61)))
         assert close(parts, ref, dtype, floor), (dtype, rel_err(parts, ref))
+
+
+def test_trace_runner_command_line(tmp_path):
+    """bin/trace_run as a user runs it: steps on standard input, `done <step>` after each, <step>.f32 for the steps that want logits;
+    two requests share steps, one ends and its pages and slot go to a third."""
+    import subprocess
+    import sys
+    import numpy as np
+    from tests.conftest import ROOT
+    cfg, w = make("all_kinds", seed=11)
+    path = write_model(tmp_path / "m", cfg, w)
+    V = cfg["vocab"]
+    ta, tb, tc = tokens(70, V, 1), tokens(9, V, 2), tokens(40, V, 3)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ta[:50], "want": [0, 49]}, {"id": "b", "tokens": tb[:8], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": tb[8:], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": ta[50:52], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "c", "tokens": tc, "want": [39]}, {"id": "a", "tokens": ta[52:], "want": [17]}], "end": ["a", "c"]}]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out", str(out),
+                        "--max-tokens", "192", "--max-live", "2"], input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+                       capture_output=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(4)]
+    assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "3.f32"]
+    read = lambda n: torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, V).copy())
+    ra, rb, rc = F.forward(cfg, w, ta), F.forward(cfg, w, tb), F.forward(cfg, w, tc)
+    assert rel_err(read(0), ra[[0, 49]]) < 1e-3 and rel_err(read(1), rb[[8]]) < 1e-3
+    assert rel_err(read(3), torch.stack([rc[39], ra[69]])) < 1e-3
