@@ -503,6 +503,11 @@ int ssd_polynorm_rows(const void* z_rows, const float* coef, float eps, void* ou
  * u = clamp(s zu, -limit, limit); out = g * sigmoid(alpha * g) * (u + 1), element-type rows [rows][F]. */
 int ssd_glu_clamp_rows(const void* ab_rows, const float* row_scale, const int32_t* perm, void* out_rows, int rows, int F, float limit,
                        float alpha, int f32, void* stream);
+/* The same clamped swish-GLU as the epilogue of the grouped product (bf16 only): w_rows [E][N][K] with the rows of every expert in
+ * (gate_i, up_i) pairs, y element-type rows [rows][N / 2]; s = row_scale ? row_scale[row_idx ? row_idx[m] : m] : 1 for sorted row m. */
+int ssd_gemm_rows_grouped_glu_clamp(const void* x_rows, const void* w_rows, void* y, const int32_t* offsets, int E,
+                                    const int32_t* row_idx, int idx_div, int rows, int N, int K, const float* row_scale, float limit,
+                                    float alpha, void* stream);
 /* fp32 logit rows in place: z = scale * z, then (cap > 0) z = cap * tanh(z / cap). */
 int ssd_logits_cap_rows(void* logits, int rows, int V, long ld, float scale, float cap, void* stream);
 /* Router of the sigmoid kind: scores = sigmoid(logits[t][0..E)) (row stride ld), the `top` largest (lowest index wins a tie) -> idx,

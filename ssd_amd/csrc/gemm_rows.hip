@@ -69,8 +69,16 @@ __device__ __forceinline__ void store_out(void* y, long row, long ldy, long n, f
 
 // epilogues 3 / 4 (bf16 forms only): the weight rows come in (gate, up) pairs -- row 2i = gate_i, row 2i + 1 = up_i -- and the output is
 // act(gate) * up as element-type rows [M][N / 2], act = silu (3) or tanh-form gelu (4).  A lane's accumulators hold both halves of a pair.
-__host__ __device__ __forceinline__ bool epi_pairs(int epi) { return epi == 3 || epi == 4; }
-__device__ __forceinline__ float glu_act(float z, float u, int epi) {
+// epilogue 6 (ssd_gemm_rows_grouped_glu_clamp): the clamped swish-GLU of experts whose routing weight multiplies their INPUT -- both
+// halves of a pair are scaled by the row's factor s = row_scale[row_idx[m]] (the products are linear in it), then g = min(s z, limit),
+// u = clamp(s u, -limit, limit), out = g sigmoid(alpha g) (u + 1).
+struct GluClamp { const float* row_scale; float limit, alpha; };
+__host__ __device__ __forceinline__ bool epi_pairs(int epi) { return epi == 3 || epi == 4 || epi == 6; }
+__device__ __forceinline__ float glu_act(float z, float u, int epi, float s = 1.0f, float limit = 0.f, float alpha = 0.f) {
+  if (epi == 6) {
+    const float g = fminf(s * z, limit);
+    return g / (1.0f + expf(-alpha * g)) * (fminf(fmaxf(s * u, -limit), limit) + 1.0f);
+  }
   const float g = epi == 3 ? z / (1.0f + expf(-z)) : 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   return g * u;
 }
@@ -79,7 +87,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
                  const int* __restrict__ offsets, int E, const int* __restrict__ row_idx, int idx_div, bool vec_ok, long ldx, long ldy,
-                 long gsx, long gsy) {
+                 long gsx, long gsy, GluClamp gc) {
   constexpr int PAD = 16 / sizeof(T);
   constexpr int LDT = BK + PAD;
   __shared__ __attribute__((aligned(16))) T sx[BM * LDT];
@@ -122,12 +130,15 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
     }
     const int m = row0 + wave * 16 + (lane & 15);
     if (m < row_end && epi_pairs(epi)) {
+      const float rs = epi == 6 && gc.row_scale ? gc.row_scale[row_idx ? row_idx[m] : m] : 1.0f;
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
         for (int r = 0; r < 4; r += 2) {
           const int n = n0 + nt * 16 + (lane >> 4) * 4 + r;
-          if (n + 1 < N) Elem<T>::st(reinterpret_cast<T*>(y) + (long)m * ldy + ycol + (n >> 1), glu_act(acc[nt][r], acc[nt][r + 1], epi));
+          if (n + 1 < N)
+            Elem<T>::st(reinterpret_cast<T*>(y) + (long)m * ldy + ycol + (n >> 1),
+                        glu_act(acc[nt][r], acc[nt][r + 1], epi, rs, gc.limit, gc.alpha));
         }
     } else if (m < row_end) {
 #pragma unroll
@@ -188,7 +199,7 @@ template <int NW>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
                    const int* __restrict__ offsets, const int* __restrict__ row_idx, int idx_div, long ldx, long ldy, long gsx,
-                   long gsy) {
+                   long gsy, GluClamp gc) {
   constexpr int U = 8;
   __shared__ f32x4_t red[NW * 64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
@@ -237,10 +248,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 #pragma unroll
       for (int wv = 1; wv < NW; ++wv) sum += red[wv * 64 + lane];
       if (mvalid && epi_pairs(epi)) {
+        const float rs = epi == 6 && gc.row_scale ? gc.row_scale[row_idx ? row_idx[mrow] : mrow] : 1.0f;
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
           const int n = n0 + qd * 4 + e;
-          if (n + 1 < N) reinterpret_cast<bf16_t*>(y)[(long)mrow * ldy + ycol + (n >> 1)] = (bf16_t)f2bf(glu_act(sum[e], sum[e + 1], epi));
+          if (n + 1 < N)
+            reinterpret_cast<bf16_t*>(y)[(long)mrow * ldy + ycol + (n >> 1)] =
+                (bf16_t)f2bf(glu_act(sum[e], sum[e + 1], epi, rs, gc.limit, gc.alpha));
         }
       } else if (mvalid) {
 #pragma unroll
@@ -257,9 +271,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 constexpr int SKINNY_MAX_ROWS = 16, SKINNY_MAX_GROUPED_ROWS = 64;
 
 int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, const int* offsets, int E, const int* row_idx,
-           int idx_div, int f32, void* stream, int G = 1, long ldx = 0, long gsx = 0, long ldy = 0, long gsy = 0) {
+           int idx_div, int f32, void* stream, int G = 1, long ldx = 0, long gsx = 0, long ldy = 0, long gsy = 0,
+           GluClamp gc = GluClamp{nullptr, 0.f, 0.f}) {
   if (!x || !w || !y) return SSD_ERR_ARG;
-  if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 5) return SSD_ERR_SHAPE;
+  if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 6) return SSD_ERR_SHAPE;
   if (epi_pairs(epi) && (f32 || (N & 1))) return SSD_ERR_SHAPE;        // the paired epilogues exist in the bf16 forms only
   if (offsets && E <= 0) return SSD_ERR_SHAPE;
   if (G < 1 || G > 65535 || (G > 1 && offsets)) return SSD_ERR_SHAPE;
@@ -278,13 +293,13 @@ int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, 
     const int kt = (K + 31) / 32;
     if (wgs < 256 && kt >= 64)
       hipLaunchKernelGGL(gemm_skinny_kernel<16>, sg, dim3(1024), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy, gc);
     else if (wgs < 1024 && kt >= 32)
       hipLaunchKernelGGL(gemm_skinny_kernel<8>, sg, dim3(512), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy, gc);
     else
       hipLaunchKernelGGL(gemm_skinny_kernel<4>, sg, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy, gc);
     return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
   }
   const int tiles_m = (M + BM - 1) / BM + (offsets ? E : 0);
@@ -293,10 +308,10 @@ int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, 
   const bool vec_ok = ((size_t)K * esz) % 16 == 0 && x_vec && ((uintptr_t)w % 16 == 0);
   if (f32)
     hipLaunchKernelGGL(gemm_rows_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, (const float*)w, y, M, N, K,
-                       epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy);
+                       epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy, gc);
   else
     hipLaunchKernelGGL(gemm_rows_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N,
-                       K, epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy);
+                       K, epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy, gc);
   return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
 }
 
@@ -312,6 +327,14 @@ extern "C" int ssd_gemm_rows_grouped(const void* x_rows, const void* w_rows, voi
                                      void* stream) {
   if (!offsets) return SSD_ERR_ARG;
   return launch(x_rows, w_rows, y, rows, N, K, epilogue, offsets, E, row_idx, idx_div, f32, stream);
+}
+
+extern "C" int ssd_gemm_rows_grouped_glu_clamp(const void* x_rows, const void* w_rows, void* y, const int32_t* offsets, int E,
+                                               const int32_t* row_idx, int idx_div, int rows, int N, int K, const float* row_scale,
+                                               float limit, float alpha, void* stream) {
+  if (!offsets) return SSD_ERR_ARG;
+  if (!(limit > 0.f)) return SSD_ERR_SHAPE;
+  return launch(x_rows, w_rows, y, rows, N, K, 6, offsets, E, row_idx, idx_div, 0, stream, 1, 0, 0, 0, 0, GluClamp{row_scale, limit, alpha});
 }
 
 extern "C" int ssd_gemm_rows_batched(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int G, long ldx, long gsx,

@@ -12,8 +12,8 @@ Launches per layer (T token rows):
     state space    W_in GEMM -> causal_conv_silu -> ssd_scan (state slot) -> group_gate_norm (gate first) -> W_o GEMM
     prenorm_tail   x += mixer output, and the feed-forward's norm
     dense ff       W_up GEMM -> polynorm_rows -> W_down GEMM
-    routed ff      router GEMM -> moe_route_sigmoid -> moe_plan -> grouped [gate | up] GEMM -> glu_clamp_rows (routing weight, clamps,
-                   swish) -> grouped W_down GEMM
+    routed ff      router GEMM -> moe_route_sigmoid -> moe_plan -> grouped [gate | up] GEMM with the clamped GLU (routing weight, clamps,
+                   swish) as epilogue (fp32 mode: + glu_clamp_rows) -> grouped W_down GEMM
     prenorm_tail   x += ff output (the routed sum rides along), and the next layer's first norm
 over pre-allocated buffers (nothing is allocated during a forward).  Same interface as ssd_amd.model.HipDecoder towards the ModelRunner.
 
@@ -94,7 +94,7 @@ class HipFomunex(Res32Decoder):
             self.r_off = z(E + 1, dtype=torch.int32)
             self.r_perm = z(T * top, dtype=torch.int32)
             self.r_inv = z(T * top, dtype=torch.int32)
-            self.ab = z(T * max(2 * m.top * m.ff for m in moes))
+            self.ab = z(T * max(2 * m.top * m.ff for m in moes)) if self.f32 else None      # bf16: the GLU is the GEMM's epilogue
             self.ydn = z(T * top * W)
         ffs = [m.ff for m in dense] + [m.top * m.ff for m in moes]
         if ffs:
@@ -159,8 +159,10 @@ class HipFomunex(Res32Decoder):
                 w[p + "mlp.up"], w[p + "mlp.down"] = cv(raw[p + "mlp.up"]), cv(raw[p + "mlp.down"])
                 w[p + "mlp.act"] = f32(raw[p + "mlp.act"])
             else:
-                w[p + "mlp.gu"] = cv(torch.stack([torch.cat([raw[p + f"mlp.e{e}.gate"], raw[p + f"mlp.e{e}.up"]], dim=0)
-                                                  for e in range(ml.experts)]))
+                # bf16: rows interleaved (gate_0, up_0, gate_1, ...) for the grouped GEMM's paired epilogue; fp32: [gate | up], the
+                # clamped GLU is a launch of its own
+                pair = (lambda g, u: torch.stack([g, u], dim=1).reshape(-1, g.shape[1])) if not self.f32 else (lambda g, u: torch.cat([g, u], dim=0))
+                w[p + "mlp.gu"] = cv(torch.stack([pair(raw[p + f"mlp.e{e}.gate"], raw[p + f"mlp.e{e}.up"]) for e in range(ml.experts)]))
                 w[p + "mlp.down"] = cv(torch.stack([raw[p + f"mlp.e{e}.down"] for e in range(ml.experts)]))
                 w[p + "mlp.router"] = cv(raw[p + "mlp.router"])
         torch.cuda.synchronize(self.device)
@@ -279,9 +281,13 @@ class HipFomunex(Res32Decoder):
         H.gemm_rows(self.hn, w[p + "router"], self.r_z, T, E, W, f)
         H.moe_route_sigmoid(self.r_z, E, self.r_idx, self.r_wt, T, E, top)
         H.moe_plan(self.r_idx, T, top, E, self.r_off, self.r_perm, self.r_inv)
-        H.gemm_rows_grouped(self.hn, w[p + "gu"], self.ab, self.r_off, E, T * top, 2 * ml.ff, W, f, H.GR_F32, row_idx=self.r_perm, idx_div=top)
         # the routing weight multiplies the expert's INPUT: both products are linear in it, so it scales their fp32 results
-        H.glu_clamp_rows(self.ab, self.act, T * top, ml.ff, ml.limit, SWISH_ALPHA, f, row_scale=self.r_wt, perm=self.r_perm)
+        if f:
+            H.gemm_rows_grouped(self.hn, w[p + "gu"], self.ab, self.r_off, E, T * top, 2 * ml.ff, W, f, H.GR_F32, row_idx=self.r_perm, idx_div=top)
+            H.glu_clamp_rows(self.ab, self.act, T * top, ml.ff, ml.limit, SWISH_ALPHA, f, row_scale=self.r_wt, perm=self.r_perm)
+        else:
+            H.gemm_rows_grouped_glu_clamp(self.hn, w[p + "gu"], self.act, self.r_off, E, T * top, 2 * ml.ff, W, ml.limit, SWISH_ALPHA,
+                                          row_idx=self.r_perm, idx_div=top, row_scale=self.r_wt)
         H.gemm_rows_grouped(self.act, w[p + "down"], self.ydn, self.r_off, E, T * top, W, ml.ff, f, H.GR_F32)
         return dict(ydn=self.ydn, inv=self.r_inv, top=top)
 

@@ -147,6 +147,8 @@ SIGNATURES = {
     "ssd_prenorm_tail": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_polynorm_rows": [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_glu_clamp_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    "ssd_gemm_rows_grouped_glu_clamp": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                        c_float, c_float, c_void_p],
     "ssd_logits_cap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_float, c_void_p],
     "ssd_moe_route_sigmoid": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_winattn_store": [c_void_p, c_long, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,

@@ -548,6 +548,13 @@ def glu_clamp_rows(ab, out_rows, rows: int, F: int, limit: float, alpha: float, 
            "ssd_glu_clamp_rows")
 
 
+def gemm_rows_grouped_glu_clamp(x, w, y, offsets, E: int, rows: int, N: int, K: int, limit: float, alpha: float, row_idx=None,
+                                idx_div: int = 1, row_scale=None):
+    """Grouped product with the clamped swish-GLU as epilogue (bf16; weight rows in (gate, up) pairs); row_scale is indexed through row_idx."""
+    _check(load_library().ssd_gemm_rows_grouped_glu_clamp(_p(x), _p(w), _p(y), _p(offsets), E, _p(row_idx), idx_div, rows, N, K,
+                                                          _p(row_scale), limit, alpha, _stream()), "ssd_gemm_rows_grouped_glu_clamp")
+
+
 def logits_cap_rows(logits, rows: int, V: int, ld: int, scale: float, cap: float):
     _check(load_library().ssd_logits_cap_rows(_p(logits), rows, V, ld, scale, cap, _stream()), "ssd_logits_cap_rows")
 

@@ -344,3 +344,31 @@ def test_grouped_gate_norm(f32, groups, gate_first):
     else:
         ref = F.rms(od.view(T, groups, -1), eps).view(T, N) * w.double() * gs
     assert torch.allclose(out.cpu().double(), ref, **tol(f32))
+
+
+@pytest.mark.parametrize("rows_per_token", [1, 3])
+@pytest.mark.parametrize("T", [5, 150])
+def test_grouped_gemm_with_the_clamped_glu_as_epilogue(T, rows_per_token):
+    """bf16: experts' [gate | up] product over rows sorted by expert, the routing weight and the clamps applied to the fp32 accumulators
+    (weight rows in (gate, up) pairs) -- few rows (the skinny form) and many (the tile form), against the two-step fp64 statement."""
+    E, W, ff, top, limit = 4, 72, 40, rows_per_token, 1.25
+    g = torch.Generator().manual_seed(T)
+    x = rnd(T, W, seed=1).to(torch.bfloat16)
+    gate, up = rnd(E, ff, W, seed=2, scale=0.3).to(torch.bfloat16), rnd(E, ff, W, seed=3, scale=0.3).to(torch.bfloat16)
+    idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    wt = torch.rand(T, top, generator=g)
+    off = torch.zeros(E + 1, dtype=torch.int32, device=DEV)
+    perm = torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    inv = torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    H().moe_plan(d(idx), T, top, E, off, perm, inv)
+    pairs = torch.stack([gate, up], dim=2).reshape(E, 2 * ff, W)
+    out = torch.zeros(T * top, ff, dtype=torch.bfloat16, device=DEV)
+    H().gemm_rows_grouped_glu_clamp(d(x), d(pairs), out, off, E, T * top, 2 * ff, W, limit, 1.702, row_idx=perm, idx_div=top, row_scale=d(wt))
+    got = out.cpu().double()[inv.cpu().long()].view(T, top, ff)
+    for t in range(T):
+        for j in range(top):
+            e, s = int(idx[t, j]), wt[t, j].double()
+            gg = torch.clamp(s * (gate[e].double() @ x[t].double()), max=limit)
+            uu = torch.clamp(s * (up[e].double() @ x[t].double()), min=-limit, max=limit)
+            ref = gg * torch.sigmoid(1.702 * gg) * (uu + 1)
+            assert torch.allclose(got[t, j], ref, rtol=2e-2, atol=2e-2), (t, j, float((got[t, j] - ref).abs().max()))
