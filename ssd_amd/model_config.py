@@ -484,6 +484,8 @@ class FomunexConfig:
     def from_json(cfg: dict) -> "FomunexConfig":
         layers = []
         for i, lc in enumerate(cfg["layers"]):
+            if "weights_of" in lc and 0 <= int(lc["weights_of"]) < len(cfg["layers"]):
+                lc = {**cfg["layers"][int(lc["weights_of"])], **lc}          # what a borrowing layer leaves out equals its source's
             m, kind = lc["mixer"], lc["type"]
             if kind == "attention":
                 mask = m.get("mask") or {}

@@ -51,6 +51,10 @@ def test_config_reader_defaults_borrowed_weights_and_sizes_from_tensor_shapes(tm
     write(tmp_path, bare, w)
     b = read_native_config(str(tmp_path))
     assert b.max_position_embeddings == 512 and (b.logit_scale, b.logit_softcap) == (1.0, 0.0) and b.layers[0].mixer.scale == 16 ** -0.5
+    short = json.loads(json.dumps(cfg))                   # a borrowing layer that only names its source: the rest equals the source's
+    short["layers"][4] = {"weights_of": 0}
+    sc = FomunexConfig.from_json(short)
+    assert sc.layers[4].mixer == sc.layers[0].mixer and sc.layers[4].mlp == sc.layers[0].mlp and sc.layers[4].weights_of == 0
     assert not FomunexConfig.from_json(F.make_config([F.attention_layer()])).recurrent
     for breakit in (lambda d: d["layers"][0].update(type="conv"), lambda d: d["layers"][0]["mlp"].update(kind="glu"),
                     lambda d: d["layers"][0]["mixer"].update(kv_heads=3), lambda d: d["layers"][1]["mlp"]["router"].update(top=9),
