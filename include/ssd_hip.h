@@ -31,7 +31,7 @@ extern "C" {
 
 /* Bumped whenever a signature or a semantic of this header changes; ssd_abi_version() returns the value the library was built
  * with, so a consumer compiled against another header can tell (tests/abi_consumer.c does). */
-#define SSD_HIP_ABI_VERSION 5
+#define SSD_HIP_ABI_VERSION 6
 
 #define SSD_OK 0
 #define SSD_ERR_SHAPE (-1)
@@ -453,7 +453,9 @@ int ssd_glu_rows(const void* ab_rows, void* out_rows, int rows, int F, int act, 
 /* Latent attention with a sliding window (csrc/attention_latent.hip).  proj_rows fp32 [T][ld] = [dq (q_rank) | latent (kv_rank) |
  * rotated key part (rot) | gate logits (H)].  Store: cq_out [T][q_rank] = rms(dq) * q_norm_w; cache row slots[t] (-1: none) of
  * cache [rows][kv_rank + rot] = [rms(latent) * kv_norm_w | rope(rotated key part)]; gate_out fp32 [T][H] = sigmoid.  rope turns the
- * first rot_dims entries (entry i pairs with i + rot_dims / 2) by positions[t] * freqs[i] with cos and sin times mag. */
+ * first rot_dims entries (entry i pairs with i + rot_dims / 2) by positions[t] * freqs[i] with cos and sin times mag.
+ * q_norm_w NULL: cq_out = the first q_rank entries as they are (queries that pass through no latent); gate_out NULL: no gates (the
+ * row then need not hold gate logits).  ssd_latent_attn: gate NULL = 1. */
 int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int kv_rank, int rot, int H, const void* q_norm_w,
                      const void* kv_norm_w, float eps, const int64_t* positions, const float* freqs, float mag, int rot_dims,
                      const int32_t* slots, void* cq_out, void* cache, void* gate_out, int T, int f32, void* stream);
@@ -472,10 +474,10 @@ int ssd_latent_attn_mfma_ok(int kv_rank, int rot, int f32);
 /* Linear attention with per-head decay over a recurrent fp32 state (csrc/lightning.hip).  proj_rows fp32 [T][ld] holds q at q_off
  * ([H][D]), k at k_off ([H][D]), v at v_off ([H][Dv]), each passed through silu.  Per sequence b (rows cu_q[b] .. cu_q[b+1]-1, or
  * q_per_seq rows each) and head: S = state[state_slots[b]][h] (zero when the first row's position is 0), per row S = decay[h] * S +
- * k v^T, out = S^T q (fp32 [T][H*Dv]); S is written back. */
+ * k v^T, out = S^T q (fp32 [T][H*Dv]); S is written back.  act 0: q, k, v = silu of the row's values; act 1: the values as they are. */
 int ssd_lightning_scan(const void* proj_rows, long ld, int q_off, int k_off, int v_off, const float* decay, const int64_t* positions,
                        const int32_t* cu_q, int q_per_seq, const int32_t* state_slots, void* state, void* out_rows, int B, int H, int D,
-                       int Dv, void* stream);
+                       int Dv, int act, void* stream);
 /* out[t] = weight * o[t] / sqrt(mean(o[t]^2) + eps) * sigmoid(proj_rows[t][g_off ..]) over N = H * Dv entries, element-type rows. */
 int ssd_lightning_gate_norm(const void* o_rows, const void* proj_rows, long ld, int g_off, const void* weight, float eps,
                             void* out_rows, int T, int N, int f32, void* stream);
@@ -508,11 +510,19 @@ int ssd_glu_clamp_rows(const void* ab_rows, const float* row_scale, const int32_
 int ssd_gemm_rows_grouped_glu_clamp(const void* x_rows, const void* w_rows, void* y, const int32_t* offsets, int E,
                                     const int32_t* row_idx, int idx_div, int rows, int N, int K, const float* row_scale, float limit,
                                     float alpha, void* stream);
+/* The dense form of the same epilogue (no groups, no row factor): y [M][N / 2] = g sigmoid(alpha g) (u + 1) of the (gate, up) row pairs. */
+int ssd_gemm_rows_glu_clamp(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, float limit, float alpha, void* stream);
 /* fp32 logit rows in place: z = scale * z, then (cap > 0) z = cap * tanh(z / cap). */
 int ssd_logits_cap_rows(void* logits, int rows, int V, long ld, float scale, float cap, void* stream);
 /* Router of the sigmoid kind: scores = sigmoid(logits[t][0..E)) (row stride ld), the `top` largest (lowest index wins a tie) -> idx,
  * weights = those scores as they are. */
 int ssd_moe_route_sigmoid(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, void* stream);
+/* The sigmoid router with a choice correction and group-limited choice: choice = sigmoid(logit) + correction[e] (NULL: 0); experts in
+ * `groups` contiguous groups, a group's score = the sum of its `group_top` (<= 8) largest choice scores, experts outside the best
+ * `keep` groups cannot be chosen (their choice score counts as -inf); the `top` largest choice scores -> idx; weights = sigmoid(logit)
+ * of the chosen, as they are. */
+int ssd_moe_route_sigmoid_grouped(const float* logits, long ld, const float* correction, int32_t* idx, float* weights, int T, int E,
+                                  int top, int groups, int keep, int group_top, void* stream);
 
 /* Sliding-window attention with unit-RMS q / k, capped scores, a per-head distance penalty and a softmax sink
  * (csrc/attention_window.hip).  Store: qkv_rows fp32 [T][ld] = [q (H*D) | k (G*D) | v (G*Dv)]; q_out [T][H*D] = q / rms(q) per head;
@@ -527,7 +537,37 @@ int ssd_winattn_store(const void* qkv_rows, long ld, float eps, const int32_t* s
 int ssd_winattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const float* slopes, const float* sinks,
                       const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq,
                       int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, int window, float scale, float cap,
-                      void* out_rows, int f32, void* stream);
+                      const float* out_freqs, void* out_rows, int f32, void* stream);
+/* The store of the rotary variant: q_out = rope(q_norm_w * q / rms(q)) with the RMS over ALL H * D entries of the row's q (k alike,
+ * over G * D, into the K cache); rope turns the first rot_dims entries of every head (entry i pairs with i + rot_dims / 2) by
+ * positions[t] * qk_freqs[i].  v_freqs (fp32 [Dv / 2], NULL: none): every value head turns over all Dv entries by positions[t] *
+ * v_freqs[i] before it is cached; ssd_winattn_paged's out_freqs (NULL: none) then turns every head's output back by the query's
+ * position (pair (m, m + Dv / 2) by -positions[t] * out_freqs[m]; the MFMA form takes Dv % 32 == 0 then). */
+int ssd_winattn_store_rope(const void* qkv_rows, long ld, const void* q_norm_w, const void* k_norm_w, float eps, const int64_t* positions,
+                           const float* qk_freqs, int rot_dims, const float* v_freqs, const int32_t* slots, void* q_out, void* k_cache,
+                           void* v_cache, int T, int H, int G, int D, int Dv, int block_size, int f32, void* stream);
+
+/* Layers that normalise a sublayer's output only, with a weighted average over the depth (csrc/postnorm.hip).
+ * ssd_embed_hist: x_out fp32 [T][W] = table[ids[t]] (zeros for an id outside the table), the same into hist0 (optional) and as
+ * element-type rows into rows_out (optional).
+ * ssd_postnorm_tail: v = y_rows[t] (fp32) or sum_j weights[t * top + j] * ydn_rows[inv[t * top + j]];  x[t] += post_weight * v /
+ * sqrt(mean(v^2) + eps) (post_weight fp32 [W]).  hist (optional, fp32 levels of hist_stride floats): level hist_levels - 1 receives
+ * x[t], then x[t] = sum_(j < hist_levels) coef[j] * level_j[t].  next_out (optional): x[t] as element-type rows.
+ * ssd_rmsnorm_w32_rows: out_rows[r] = weight * x[g] / sqrt(mean(x[g]^2) + eps), g = gather[r] or r; weight fp32.
+ * ssd_rope_rows: in place on fp32 rows [T][ld]: blocks of `heads` heads of D entries at columns off_a and off_b (off_b < 0: one block);
+ * the first rot_dims entries of a head turn (entry i pairs with i + rot_dims / 2) by positions[t] * freqs[i], then the head is
+ * multiplied by the block's scale.
+ * ssd_gate_rows: out_rows[t][c] = o_rows[t * ldo + c] * sigmoid(gate_rows[t * ldg + c]) for c < N, element-type rows out. */
+int ssd_embed_hist(const int64_t* ids, const void* table, void* x_out, void* hist0, void* rows_out, int T, int W, long vocab, int f32,
+                   void* stream);
+int ssd_postnorm_tail(const void* y_rows, const void* ydn_rows, const int32_t* inv, const float* weights, int top,
+                      const float* post_weight, float eps, void* x, void* hist, long hist_stride, int hist_levels, const float* coef,
+                      void* next_out, int T, int W, int f32, void* stream);
+int ssd_rmsnorm_w32_rows(const void* x, const float* weight, float eps, void* out_rows, const int32_t* gather, int T, int W, int f32,
+                         void* stream);
+int ssd_rope_rows(void* rows, long ld, const int64_t* positions, const float* freqs, int rot_dims, int heads, int D, int off_a,
+                  float scale_a, int off_b, float scale_b, int T, void* stream);
+int ssd_gate_rows(const void* o_rows, long ldo, const void* gate_rows, long ldg, void* out_rows, int T, int N, int f32, void* stream);
 
 /* Recurrent mixers over per-sequence state slots (csrc/recurrent.hip).  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows
  * each; state_slots int32 [B]; a sequence whose first row has position 0 starts from zero whatever its slot holds.

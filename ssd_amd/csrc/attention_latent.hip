@@ -10,6 +10,7 @@
 // Rotation: the first `rot_dims` of the R rotated entries turn, entry i pairing with i + rot_dims / 2, by angle p * f_i (fp32) with
 // cos and sin scaled by `mag`; f and mag come from the host (they carry the YaRN frequency blend).
 //  * ssd_latent_store  fp32 projection rows [dq | dkv | gate logits] -> c_q rows, the cache row of every token, sigmoid gates
+//                      (no q norm weight: the first q_rank entries pass as they are -- queries without a latent; no gate_out: no gates)
 //  * ssd_latent_attn   MFMA form below (bf16, aligned latent sizes), else the scalar fp32 form for any sizes and both element types: a wave owns a (token, head) row, a lane a key for the
 //                      scores and latent columns for the weighted sum; keys in steps of 64 from the window's first key, so a row's
 //                      arithmetic depends on its position alone (not on the portion or the batch it arrives in)
@@ -69,8 +70,13 @@ latent_store_kernel(const float* __restrict__ proj, long ld, int Qr, int Cr, int
   sq = block_sum_256(sq, red);
   sc = block_sum_256(sc, red);
   const float rq = 1.0f / sqrtf(sq / (float)Qr + eps), rc = 1.0f / sqrtf(sc / (float)Cr + eps);
-  for (int i = threadIdx.x; i < Qr; i += 256) stf<T>(cq_out + t * Qr + i, dq[i] * rq * ldf<T>(wq + i));
-  for (int i = threadIdx.x; i < H; i += 256) gate_out[t * H + i] = sigmoidf_(pr[Qr + Cr + R + i]);
+  if (wq) {
+    for (int i = threadIdx.x; i < Qr; i += 256) stf<T>(cq_out + t * Qr + i, dq[i] * rq * ldf<T>(wq + i));
+  } else {                                            // queries that pass through no latent: the first Qr entries as they are
+    for (int i = threadIdx.x; i < Qr; i += 256) stf<T>(cq_out + t * Qr + i, dq[i]);
+  }
+  if (gate_out)
+    for (int i = threadIdx.x; i < H; i += 256) gate_out[t * H + i] = sigmoidf_(pr[Qr + Cr + R + i]);
   const int slot = slots[t];
   if (slot < 0) return;
   T* row = cache + (size_t)slot * (Cr + R);
@@ -151,7 +157,7 @@ latent_attn_kernel(const float* __restrict__ q_abs, const T* __restrict__ q_rows
       }
     }
   }
-  const float g = gate[(size_t)t * H + h] / den;
+  const float g = (gate ? gate[(size_t)t * H + h] : 1.0f) / den;
 #pragma unroll
   for (int c = 0; c < LAT_MAXC; ++c) {
     const int col = lane + 64 * c;
@@ -320,7 +326,7 @@ latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restri
     return;
   }
   if (!hv) return;
-  const float gsc = gate[(size_t)t * H + h] / Dn;
+  const float gsc = (gate ? gate[(size_t)t * H + h] : 1.0f) / Dn;
   for (int nt = wave; nt < NT; nt += NW) {
     float v[4];
 #pragma unroll
@@ -356,7 +362,7 @@ latent_attn_merge_kernel(const float* __restrict__ ws, const float* __restrict__
     Dn += u[z * unit + (size_t)Cr * 16 + 16 + i] * fz;
     a += u[z * unit + idx] * fz;
   }
-  out[((size_t)t * H + h) * Cr + col] = (bf16_t)f2bf(a * (gate[(size_t)t * H + h] / Dn));
+  out[((size_t)t * H + h) * Cr + col] = (bf16_t)f2bf(a * ((gate ? gate[(size_t)t * H + h] : 1.0f) / Dn));
 }
 
 static inline bool latent_mfma_ok(int Cr, int R) {
@@ -371,9 +377,9 @@ extern "C" int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int 
                                 const void* kv_norm_w, float eps, const int64_t* positions, const float* freqs, float mag,
                                 int rot_dims, const int32_t* slots, void* cq_out, void* cache, void* gate_out, int T, int f32,
                                 void* stream) {
-  if (!proj_rows || !q_norm_w || !kv_norm_w || !positions || !freqs || !slots || !cq_out || !cache || !gate_out) return SSD_ERR_ARG;
+  if (!proj_rows || !kv_norm_w || !positions || !freqs || !slots || !cq_out || !cache) return SSD_ERR_ARG;
   if (T <= 0 || q_rank <= 0 || kv_rank <= 0 || rot < 0 || H <= 0 || rot_dims < 0 || rot_dims > rot || (rot_dims & 1) ||
-      ld < (long)q_rank + kv_rank + rot + H)
+      ld < (long)q_rank + kv_rank + rot + (gate_out ? H : 0))
     return SSD_ERR_SHAPE;
   if (f32)
     hipLaunchKernelGGL(latent_store_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_rank,
@@ -391,7 +397,7 @@ extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void
                                int rot, int kv_rank, int block_size, int window, float scale, const float* freqs, float mag,
                                int rot_dims, void* out_rows, int f32, int q_abs_elem, void* workspace, long workspace_bytes,
                                void* stream) {
-  if (!q_abs || !q_rows || !cache || !gate || !block_tables || !positions || !freqs || !out_rows) return SSD_ERR_ARG;
+  if (!q_abs || !q_rows || !cache || !block_tables || !positions || !freqs || !out_rows) return SSD_ERR_ARG;
   if (B <= 0 || T <= 0 || H <= 0 || D <= 0 || rot < 0 || kv_rank <= 0 || kv_rank > 64 * LAT_MAXC || block_size <= 0 || max_blocks <= 0 ||
       rot_dims < 0 || rot_dims > rot || (rot_dims & 1) || (!cu_q && q_per_seq <= 0))
     return SSD_ERR_SHAPE;

@@ -13,6 +13,11 @@
 //                         wave order, then the sink joins the denominator.
 //                         MFMA form (bf16, D % 32 == 0, D <= 256, Dv % 16 == 0, Dv <= 256, block_size % 32 == 0; the caller gives
 //                         max_q, an upper bound of the rows a sequence brings): see below.
+//   * ssd_winattn_store_rope  the store of a rotary variant: RMS norm with weights over the WHOLE q and the whole k projection (before
+//                         the heads are split), rotary positions on the first rot_dims entries of every q / k head, and (v_freqs given)
+//                         every value head turned by its own position over all Dv entries before it is cached; the attention then
+//                         turns every head's output back by the query's position (out_freqs), so that the weighted sum carries
+//                         relative positions.  Pairs are (i, i + n / 2) throughout.
 //   Scores, weights, sums and norms are fp32 whatever the element type.  A token's position and sequence come from positions[] and
 //   cu_q[] (varlen batches: prompt portions beside single tokens) or q_per_seq (fixed rows per sequence).
 #include "common.h"
@@ -62,6 +67,71 @@ winattn_store_kernel(const float* __restrict__ qkv, long ld, float eps, const in
   }
 }
 
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// One workgroup per token.  q' = w_q * q / rms(q) over all H * D entries (k alike over G * D), then per head the pair (i, i + half)
+// turns by pos * qk_freqs[i]; v heads turn over all Dv entries by pos * v_freqs[i] (v_freqs NULL: stored as they are).
+template <typename T>
+__global__ void __launch_bounds__(256)
+winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __restrict__ wq, const T* __restrict__ wk, float eps,
+                          const int64_t* __restrict__ positions, const float* __restrict__ qk_freqs, int rot_dims,
+                          const float* __restrict__ v_freqs, const int32_t* __restrict__ slots, T* __restrict__ q_out,
+                          T* __restrict__ kc, T* __restrict__ vc, int H, int G, int D, int Dv, int bs) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const int Nq = H * D, Nk = G * D, Nv = G * Dv;
+  const float* row = qkv + (size_t)t * ld;
+  const float pos = (float)positions[t];
+  const int slot = slots[t];
+  const long blk = slot >= 0 ? slot / bs : 0;
+  const int off = slot >= 0 ? slot % bs : 0;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < Nq; i += 256) { const float v = row[i]; sq += v * v; }
+  for (int i = threadIdx.x; i < Nk; i += 256) { const float v = row[Nq + i]; sk += v * v; }
+  sq = block_sum_256(sq, red);
+  sk = block_sum_256(sk, red);
+  const float rq = 1.0f / sqrtf(sq / (float)Nq + eps), rk = 1.0f / sqrtf(sk / (float)Nk + eps);
+  const int half = rot_dims >> 1;
+  for (int i = threadIdx.x; i < Nq + Nk; i += 256) {
+    const bool isq = i < Nq;
+    const int j = isq ? i : i - Nq, d = j % D;
+    const float* src = row + (isq ? 0 : Nq);
+    const T* w = isq ? wq : wk;
+    const float r = isq ? rq : rk;
+    float v = src[j] * r * ldf<T>(w + j);
+    if (d < rot_dims) {
+      const int f = d < half ? d : d - half;
+      const int jp = d < half ? j + half : j - half;
+      const float o = src[jp] * r * ldf<T>(w + jp);
+      const float ang = pos * qk_freqs[f];
+      const float c = cosf(ang), sn = sinf(ang);
+      v = d < half ? v * c - o * sn : v * c + o * sn;
+    }
+    if (isq) stf<T>(q_out + (size_t)t * Nq + j, v);
+    else if (slot >= 0) stf<T>(kc + (((size_t)blk * G + j / D) * bs + off) * D + d, v);
+  }
+  if (slot < 0) return;
+  const int hv = Dv >> 1;
+  for (int cI = threadIdx.x; cI < Nv; cI += 256) {
+    const int g = cI / Dv, d = cI % Dv;
+    float v = row[Nq + Nk + cI];
+    if (v_freqs) {
+      const int f = d < hv ? d : d - hv;
+      const float o = row[Nq + Nk + (d < hv ? cI + hv : cI - hv)];
+      const float ang = pos * v_freqs[f];
+      const float c = cosf(ang), sn = sinf(ang);
+      v = d < hv ? v * c - o * sn : v * c + o * sn;
+    }
+    stf<T>(vc + (((size_t)blk * G + g) * Dv + d) * bs + off, v);
+  }
+}
+
 __device__ __forceinline__ int seq_of_row(const int32_t* cu_q, int q_per_seq, int B, int t) {
   if (!cu_q) return t / q_per_seq;
   int lo = 0, hi = B;
@@ -74,7 +144,7 @@ __global__ void __launch_bounds__(256)
 winattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc, const float* __restrict__ slopes,
                      const float* __restrict__ sinks, const int32_t* __restrict__ bt, int max_blocks,
                      const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq, int B, int H, int G, int D,
-                     int Dv, int bs, int window, float scale, float cap, T* __restrict__ out) {
+                     int Dv, int bs, int window, float scale, float cap, const float* __restrict__ out_freqs, T* __restrict__ out) {
   extern __shared__ float smem[];
   const int t = blockIdx.x, h = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int g = h / (H / G);
@@ -153,10 +223,21 @@ winattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T*
     f[w] = sml[w * 2 + 1] > 0.f ? expf(sml[w * 2] - M) : 0.f;
     L += sml[w * 2 + 1] * f[w];
   }
+  const int hv = Dv >> 1;
   for (int d = threadIdx.x; d < Dv; d += 256) {
     float s = 0.f;
     for (int w = 0; w < 4; ++w) s += sacc[w * Dv + d] * f[w];
-    stf<T>(out + ((size_t)t * H + h) * Dv + d, s / L);
+    s = s / L;
+    if (out_freqs) {                  // the head's output turns back by the query's position: pair (m, m + Dv / 2) by -pos * freq[m]
+      const int dp = d < hv ? d + hv : d - hv;
+      float o = 0.f;
+      for (int w = 0; w < 4; ++w) o += sacc[w * Dv + dp] * f[w];
+      o = o / L;
+      const float ang = (float)pos * out_freqs[d < hv ? d : d - hv];
+      const float c = cosf(ang), sn = sinf(ang);
+      s = d < hv ? s * c + o * sn : s * c - o * sn;
+    }
+    stf<T>(out + ((size_t)t * H + h) * Dv + d, s);
   }
 }
 
@@ -181,7 +262,7 @@ __global__ void __launch_bounds__(256)
 winattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vt,
                     const float* __restrict__ slopes, const float* __restrict__ sinks, const int32_t* __restrict__ bt, int max_blocks,
                     const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq, int H, int G, int D, int Dv,
-                    int bs, int window, float scale, float cap, bf16_t* __restrict__ out) {
+                    int bs, int window, float scale, float cap, const float* __restrict__ out_freqs, bf16_t* __restrict__ out) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
   const int b = blockIdx.z, g = blockIdx.y, R = H / G;
@@ -337,13 +418,52 @@ winattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
   const float fo = ls > 0.f ? __expf(mx - M) : 0.f;
   const float den = ls * fo + (sinks ? __expf(sink - M) : 0.f);
   const float rs = fo / den;
+#pragma unroll
+  for (int i = 0; i < MV; ++i)
+    if (i < DVT) acc[i] *= rs;
+  if (out_freqs) {
+    // the head's output turns back by the query's position; Dv % 32 == 0 here, so the partner of column i * 16 + qd * 4 + e (the
+    // column Dv / 2 further) is element e of tile i + DVT / 2 of the SAME lane
+    const int HT = DVT >> 1;
+    if (DVT == MV) {
+#pragma unroll
+      for (int i = 0; i < MV / 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float ang = (float)pos * out_freqs[i * 16 + qd * 4 + e];
+          const float c = cosf(ang), sn = sinf(ang);
+          const float a = acc[i][e], b = acc[i + MV / 2][e];
+          acc[i][e] = a * c + b * sn;
+          acc[i + MV / 2][e] = b * c - a * sn;
+        }
+    } else {          // fewer value tiles than the register array holds: the partner tile's index is not a constant; select it
+#pragma unroll
+      for (int i = 0; i < MV / 2; ++i)
+        if (i < HT) {
+          f32x4_t pb = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int k = 0; k < MV; ++k) pb = (k == i + HT) ? acc[k] : pb;
+          f32x4_t na, nb;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float ang = (float)pos * out_freqs[i * 16 + qd * 4 + e];
+            const float c = cosf(ang), sn = sinf(ang);
+            na[e] = acc[i][e] * c + pb[e] * sn;
+            nb[e] = pb[e] * c - acc[i][e] * sn;
+          }
+          acc[i] = na;
+#pragma unroll
+          for (int k = 0; k < MV; ++k) acc[k] = (k == i + HT) ? nb : acc[k];
+        }
+    }
+  }
   bf16_t* orow = out + ((size_t)token * H + head) * Dv + qd * 4;
 #pragma unroll
   for (int i = 0; i < MV; ++i)
     if (i < DVT) {
       u32x2_t o2;
-      o2[0] = pack_bf2_hw(acc[i][0] * rs, acc[i][1] * rs);
-      o2[1] = pack_bf2_hw(acc[i][2] * rs, acc[i][3] * rs);
+      o2[0] = pack_bf2_hw(acc[i][0], acc[i][1]);
+      o2[1] = pack_bf2_hw(acc[i][2], acc[i][3]);
       *reinterpret_cast<u32x2_t*>(orow + i * 16) = o2;
     }
 }
@@ -368,22 +488,43 @@ extern "C" int ssd_winattn_store(const void* qkv_rows, long ld, float eps, const
   return LAUNCH_OK();
 }
 
+extern "C" int ssd_winattn_store_rope(const void* qkv_rows, long ld, const void* q_norm_w, const void* k_norm_w, float eps,
+                                      const int64_t* positions, const float* qk_freqs, int rot_dims, const float* v_freqs,
+                                      const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int T, int H, int G, int D, int Dv,
+                                      int block_size, int f32, void* stream) {
+  if (!qkv_rows || !q_norm_w || !k_norm_w || !positions || !slots || !q_out || !k_cache || !v_cache || (rot_dims > 0 && !qk_freqs))
+    return SSD_ERR_ARG;
+  if (T <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || block_size <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1) ||
+      (v_freqs && (Dv & 1)) || ld < (long)(H + G) * D + (long)G * Dv)
+    return SSD_ERR_SHAPE;
+  if (f32)
+    hipLaunchKernelGGL(winattn_store_rope_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
+                       (const float*)q_norm_w, (const float*)k_norm_w, eps, positions, qk_freqs, rot_dims, v_freqs, slots,
+                       (float*)q_out, (float*)k_cache, (float*)v_cache, H, G, D, Dv, block_size);
+  else
+    hipLaunchKernelGGL(winattn_store_rope_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
+                       (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, positions, qk_freqs, rot_dims, v_freqs, slots,
+                       (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, block_size);
+  return LAUNCH_OK();
+}
+
 extern "C" int ssd_winattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const float* slopes, const float* sinks,
                                  const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q,
                                  int q_per_seq, int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, int window,
-                                 float scale, float cap, void* out_rows, int f32, void* stream) {
+                                 float scale, float cap, const float* out_freqs, void* out_rows, int f32, void* stream) {
   if (!q_rows || !k_cache || !v_cache || !block_tables || !positions || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * WA_MAXV || block_size <= 0 || window < 0 ||
-      max_blocks <= 0 || (!cu_q && q_per_seq <= 0) || H > 65535)
+      max_blocks <= 0 || (!cu_q && q_per_seq <= 0) || H > 65535 || (out_freqs && (Dv & 1)))
     return SSD_ERR_SHAPE;
-  if (!f32 && max_q > 0 && D % 32 == 0 && D <= 256 && Dv % 16 == 0 && Dv <= 256 && block_size % 32 == 0 && G <= 65535 && B <= 65535) {
+  if (!f32 && max_q > 0 && D % 32 == 0 && D <= 256 && Dv % (out_freqs ? 32 : 16) == 0 && Dv <= 256 && block_size % 32 == 0 && G <= 65535 &&
+      B <= 65535) {
     const int R = H / G;
     const dim3 grid((unsigned)(((long)max_q * R + 63) / 64), G, B);
     const size_t lds = (4 * 16 * (size_t)Dv + 128) * sizeof(float);
 #define WIN_MFMA(MK, MV)                                                                                                            \
   hipLaunchKernelGGL((winattn_mfma_kernel<MK, MV>), grid, dim3(256), lds, (hipStream_t)stream, (const bf16_t*)q_rows,               \
                      (const bf16_t*)k_cache, (const bf16_t*)v_cache, slopes, sinks, block_tables, max_blocks, positions, cu_q,      \
-                     q_per_seq, H, G, D, Dv, block_size, window, scale, cap, (bf16_t*)out_rows)
+                     q_per_seq, H, G, D, Dv, block_size, window, scale, cap, out_freqs, (bf16_t*)out_rows)
     if (D <= 64 && Dv <= 64) WIN_MFMA(2, 4);
     else if (D <= 128 && Dv <= 128) WIN_MFMA(4, 8);
     else {
@@ -400,10 +541,10 @@ extern "C" int ssd_winattn_paged(const void* q_rows, const void* k_cache, const 
   if (f32)
     hipLaunchKernelGGL(winattn_paged_kernel<float>, dim3(T, H), dim3(256), bytes, (hipStream_t)stream, (const float*)q_rows,
                        (const float*)k_cache, (const float*)v_cache, slopes, sinks, block_tables, max_blocks, positions, cu_q, q_per_seq,
-                       B, H, G, D, Dv, block_size, window, scale, cap, (float*)out_rows);
+                       B, H, G, D, Dv, block_size, window, scale, cap, out_freqs, (float*)out_rows);
   else
     hipLaunchKernelGGL(winattn_paged_kernel<bf16_t>, dim3(T, H), dim3(256), bytes, (hipStream_t)stream, (const bf16_t*)q_rows,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, slopes, sinks, block_tables, max_blocks, positions, cu_q,
-                       q_per_seq, B, H, G, D, Dv, block_size, window, scale, cap, (bf16_t*)out_rows);
+                       q_per_seq, B, H, G, D, Dv, block_size, window, scale, cap, out_freqs, (bf16_t*)out_rows);
   return LAUNCH_OK();
 }

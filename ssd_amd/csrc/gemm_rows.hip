@@ -337,6 +337,12 @@ extern "C" int ssd_gemm_rows_grouped_glu_clamp(const void* x_rows, const void* w
   return launch(x_rows, w_rows, y, rows, N, K, 6, offsets, E, row_idx, idx_div, 0, stream, 1, 0, 0, 0, 0, GluClamp{row_scale, limit, alpha});
 }
 
+extern "C" int ssd_gemm_rows_glu_clamp(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, float limit, float alpha,
+                                       void* stream) {
+  if (!(limit > 0.f)) return SSD_ERR_SHAPE;
+  return launch(x_rows, w_rows, y, M, N, K, 6, nullptr, 0, nullptr, 1, 0, stream, 1, 0, 0, 0, 0, GluClamp{nullptr, limit, alpha});
+}
+
 extern "C" int ssd_gemm_rows_batched(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int G, long ldx, long gsx,
                                      long ldy, long gsy, int epilogue, int f32, void* stream) {
   if (ldx <= 0 || ldy <= 0 || gsx < 0 || gsy < 0) return SSD_ERR_SHAPE;

@@ -1,7 +1,8 @@
 // Linear attention with a per-head scalar decay over a recurrent fp32 state ("lightning" mixers):
 //     S_t = decay_h * S_(t-1) + k_t v_t^T        (S: [D][Dv] per sequence and head, zero before position 0)
 //     o_t = S_t^T q_t
-// q, k, v = silu of the projection rows.  The state of a live sequence sits in a slot of a per-layer-run pool
+// q, k, v = silu of the projection rows (act 0), or the rows as they are (act 1: a mixer that prepared them itself, e.g. rotated q / k
+// of a retention layer).  The state of a live sequence sits in a slot of a per-layer-run pool
 // state[slots][H][D][Dv] (fp32); a forward reads the slot unless the rows it brings start at position 0, walks its rows in order and
 // writes the slot back, so a prompt may arrive in portions of any size and decoding is the one-row case of the same kernel.
 //  * ssd_lightning_scan       proj rows fp32 [T][ld] holding [q | k | v | ...] -> o fp32 [T][H*Dv], state updated in place
@@ -29,7 +30,7 @@ __global__ void __launch_bounds__(256)
 lightning_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
                       const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
                       const int32_t* __restrict__ state_slots, float* __restrict__ state, float* __restrict__ out, int H, int D, int Dv,
-                      int EP) {
+                      int EP, int raw) {
   extern __shared__ float lds[];
   float* S = lds;                         // [D][Dv]
   float* sq = S + (size_t)D * Dv;         // [D]
@@ -50,10 +51,11 @@ lightning_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_
     const float* pr = proj + (size_t)r * ld;
     __syncthreads();                      // the previous row's readers of sq / sk / sv / po are done; S is loaded
     for (int i = tid; i < D; i += 256) {
-      sq[i] = siluf_(pr[q_off + h * D + i]);
-      sk[i] = siluf_(pr[k_off + h * D + i]);
+      const float qv = pr[q_off + h * D + i], kv = pr[k_off + h * D + i];
+      sq[i] = raw ? qv : siluf_(qv);
+      sk[i] = raw ? kv : siluf_(kv);
     }
-    for (int i = tid; i < Dv; i += 256) sv[i] = siluf_(pr[v_off + h * Dv + i]);
+    for (int i = tid; i < Dv; i += 256) { const float vv = pr[v_off + h * Dv + i]; sv[i] = raw ? vv : siluf_(vv); }
     __syncthreads();
     for (int e = el; e < Dv; e += EP) {
       const float ve = sv[e];
@@ -81,7 +83,7 @@ lightning_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_
 // eight at a time (silu applied once), every thread then walks the eight tokens without a barrier (it touches only its own state and
 // the staged rows), and the eight d-groups' partial outputs are summed in group order.  The arithmetic of a row is the same for any
 // portioning: the per-element chain in token order, the output sum over n ascending, then over g ascending.
-template <int EPT>
+template <int EPT, bool RAW>
 __global__ void __launch_bounds__(256)
 lightning_scan_reg_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
                           const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
@@ -126,10 +128,10 @@ lightning_scan_reg_kernel(const float* __restrict__ proj, long ld, int q_off, in
 #pragma unroll
     for (int c = 0; c < QK; ++c) {
       const int idx = tid + 256 * c;
-      sq[idx / D][idx % D] = siluf_(rq[c]);
-      sk[idx / D][idx % D] = siluf_(rk[c]);
+      sq[idx / D][idx % D] = RAW ? rq[c] : siluf_(rq[c]);
+      sk[idx / D][idx % D] = RAW ? rk[c] : siluf_(rk[c]);
     }
-    sv[g][e] = siluf_(rv);
+    sv[g][e] = RAW ? rv : siluf_(rv);
     __syncthreads();
     if (r + TB < row1) fetch(r + TB);
     for (int tt = 0; tt < nb; ++tt) {
@@ -180,19 +182,22 @@ lightning_gate_norm_kernel(const float* __restrict__ o, const float* __restrict_
 
 extern "C" int ssd_lightning_scan(const void* proj_rows, long ld, int q_off, int k_off, int v_off, const float* decay,
                                   const int64_t* positions, const int32_t* cu_q, int q_per_seq, const int32_t* state_slots,
-                                  void* state, void* out_rows, int B, int H, int D, int Dv, void* stream) {
+                                  void* state, void* out_rows, int B, int H, int D, int Dv, int act, void* stream) {
   if (!proj_rows || !decay || !positions || !state_slots || !state || !out_rows) return SSD_ERR_ARG;
-  if (B <= 0 || H <= 0 || D <= 0 || Dv <= 0 || (!cu_q && q_per_seq <= 0)) return SSD_ERR_SHAPE;
+  if (B <= 0 || H <= 0 || D <= 0 || Dv <= 0 || (!cu_q && q_per_seq <= 0) || act < 0 || act > 1) return SSD_ERR_SHAPE;
   if (Dv % 32 == 0 && Dv / 32 <= 65535 && (D == 32 || D == 64 || D == 128 || D == 256)) {
     const dim3 grid(B, H, Dv / 32);
+#define SCAN_REG1(EPT, RAW)                                                                                                        \
+  hipLaunchKernelGGL((lightning_scan_reg_kernel<EPT, RAW>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld,  \
+                     q_off, k_off, v_off, decay, positions, cu_q, q_per_seq, state_slots, (float*)state, (float*)out_rows, H, Dv)
 #define SCAN_REG(EPT)                                                                                                              \
-  hipLaunchKernelGGL(lightning_scan_reg_kernel<EPT>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_off,  \
-                     k_off, v_off, decay, positions, cu_q, q_per_seq, state_slots, (float*)state, (float*)out_rows, H, Dv)
+  do { if (act) SCAN_REG1(EPT, true); else SCAN_REG1(EPT, false); } while (0)
     if (D == 32) SCAN_REG(4);
     else if (D == 64) SCAN_REG(8);
     else if (D == 128) SCAN_REG(16);
     else SCAN_REG(32);
 #undef SCAN_REG
+#undef SCAN_REG1
     return LAUNCH_OK();
   }
   int EP = 1;
@@ -203,7 +208,7 @@ extern "C" int ssd_lightning_scan(const void* proj_rows, long ld, int q_off, int
       hipFuncSetAttribute((const void*)lightning_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
     return SSD_ERR_LAUNCH;
   hipLaunchKernelGGL(lightning_scan_kernel, dim3(B, H), dim3(256), bytes, (hipStream_t)stream, (const float*)proj_rows, ld, q_off, k_off,
-                     v_off, decay, positions, cu_q, q_per_seq, state_slots, (float*)state, (float*)out_rows, H, D, Dv, EP);
+                     v_off, decay, positions, cu_q, q_per_seq, state_slots, (float*)state, (float*)out_rows, H, D, Dv, EP, act);
   return LAUNCH_OK();
 }
 

@@ -5,6 +5,9 @@
 //                    best `keep` (by their largest score) stay eligible, the `top` largest eligible scores, divided by their sum
 //                    (+ 1e-20) and multiplied by a constant
 //   ssd_moe_route_sigmoid  scores = sigmoid of the logits, the `top` largest, weights = those scores unrenormalised
+//   ssd_moe_route_sigmoid_grouped  sigmoid scores with a per-expert correction that enters the CHOICE only: choice = score + correction;
+//                    experts in contiguous groups, a group's score = the sum of its `group_top` largest choice scores, only the best
+//                    `keep` groups stay eligible; the `top` largest eligible choice scores win; weights = the chosen experts' plain scores
 //   ssd_moe_plan     counting sort of the T * top (token, slot) pairs by expert: offsets[E+1], perm (sorted row -> pair), inv (pair -> sorted row)
 //   ssd_moe_combine  out[t] = sum_j weight[t][j] * y[inv[t * top + j]] (+ shared[t]) in slot order, fp32
 // Between plan and combine the caller runs the experts as two grouped GEMMs over the sorted rows (up with the activation as epilogue,
@@ -122,6 +125,75 @@ moe_route_sigmoid_kernel(const float* __restrict__ zin, long ldz, int32_t* __res
   if (lane < top) wt[(size_t)t * top + lane] = myval;
 }
 
+// Sigmoid routing with a choice correction and group-limited choice.  One wave per token.  Choice scores may be negative, so an
+// expert that cannot be chosen is marked by -inf (never by a finite number).  Among equal values the lowest index wins.
+constexpr int MOE_MAX_GROUP_TOP = 8;
+
+__global__ void __launch_bounds__(64)
+moe_route_sigmoid_grouped_kernel(const float* __restrict__ zin, long ldz, const float* __restrict__ corr, int32_t* __restrict__ idx,
+                                 float* __restrict__ wt, int E, int top, int groups, int keep, int group_top) {
+  extern __shared__ float z[];      // [E] scores, [E] choice scores, [groups] group scores
+  float* ch = z + E;
+  float* gs = ch + E;
+  const int t = blockIdx.x, lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) {
+    const float sc = 1.0f / (1.0f + expf(-zin[(size_t)t * ldz + e]));
+    z[e] = sc;
+    ch[e] = sc + (corr ? corr[e] : 0.f);
+  }
+  __syncthreads();
+  if (groups > 1 && keep < groups) {
+    const int per = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+      int taken[MOE_MAX_GROUP_TOP];
+      float sum = 0.f;
+      for (int j = 0; j < group_top && j < per; ++j) {
+        float b = -INFINITY; int bi = -1;
+        for (int i = 0; i < per; ++i) {
+          bool used = false;
+          for (int q = 0; q < j; ++q) used |= taken[q] == i;
+          const float v = ch[g * per + i];
+          if (!used && (bi < 0 || v > b)) { b = v; bi = i; }
+        }
+        taken[j] = bi;
+        sum += b;
+      }
+      gs[g] = sum;
+    }
+    __syncthreads();
+    // `keep` rounds of a wave-wide argmax over the groups; a kept group is marked by +inf
+    for (int j = 0; j < keep; ++j) {
+      float best = -INFINITY; int bi = 0x7fffffff;
+      for (int g = lane; g < groups; g += 64) { const float v = gs[g]; if (v != INFINITY && (bi == 0x7fffffff || v > best)) { best = v; bi = g; } }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+      }
+      if (lane == 0 && bi != 0x7fffffff) gs[bi] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < E; e += 64) if (gs[e / per] != INFINITY) ch[e] = -INFINITY;
+    __syncthreads();
+  }
+  float myval = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY; int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) { const float v = ch[e]; if (v > best) { best = v; bi = e; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if (bi == 0x7fffffff) bi = 0;       // (unreachable for finite logits: top <= eligible experts)
+    if (lane == j % 64) { myval = z[bi]; idx[(size_t)t * top + j] = bi; }
+    __syncthreads();
+    if (lane == 0) ch[bi] = -INFINITY;
+    __syncthreads();
+  }
+  if (lane < top) wt[(size_t)t * top + lane] = myval;
+}
+
 __global__ void __launch_bounds__(1024)
 moe_plan_kernel(const int32_t* __restrict__ idx, int n, int E, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
                 int32_t* __restrict__ inv) {
@@ -181,6 +253,17 @@ extern "C" int ssd_moe_route_sigmoid(const float* logits, long ld, int32_t* idx,
   if (!logits || !idx || !weights) return SSD_ERR_ARG;
   if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > E || top > MOE_MAX_TOP || ld < E) return SSD_ERR_SHAPE;
   hipLaunchKernelGGL(moe_route_sigmoid_kernel, dim3(T), dim3(64), E * sizeof(float), (hipStream_t)stream, logits, ld, idx, weights, E, top);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_moe_route_sigmoid_grouped(const float* logits, long ld, const float* correction, int32_t* idx, float* weights, int T,
+                                             int E, int top, int groups, int keep, int group_top, void* stream) {
+  if (!logits || !idx || !weights) return SSD_ERR_ARG;
+  if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > MOE_MAX_TOP || ld < E || groups <= 0 || E % groups || keep <= 0 ||
+      keep > groups || top > (E / groups) * keep || group_top <= 0 || group_top > MOE_MAX_GROUP_TOP)
+    return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_sigmoid_grouped_kernel, dim3(T), dim3(64), (2 * E + groups) * sizeof(float), (hipStream_t)stream, logits,
+                     ld, correction, idx, weights, E, top, groups, keep, group_top);
   return LAUNCH_OK();
 }
 

@@ -40,6 +40,9 @@ def model_class(family: str):
     if family == "fomunex":
         from ssd_amd.fomunex import HipFomunex
         return HipFomunex
+    if family == "dosuvik":
+        from ssd_amd.dosuvik import HipDosuvik
+        return HipDosuvik
     return HipDecoder
 
 

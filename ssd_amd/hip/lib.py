@@ -16,7 +16,7 @@ _LIB = None
 
 c_void_p, c_int, c_long, c_float, c_int64 = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_int64
 
-ABI_VERSION = 5       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
+ABI_VERSION = 6       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
 
 # name -> argtypes, exactly include/ssd_hip.h (+ include/ssd_hip_tune.h)
 SIGNATURES = {
@@ -139,7 +139,7 @@ SIGNATURES = {
                         c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p],
     "ssd_latent_attn_mfma_ok": [c_int, c_int, c_int],
     "ssd_lightning_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                           c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ssd_lightning_gate_norm": [c_void_p, c_void_p, c_long, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_moe_route_softmax": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ssd_embed_pos_res32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_long, c_long,
@@ -154,7 +154,17 @@ SIGNATURES = {
     "ssd_winattn_store": [c_void_p, c_long, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
     "ssd_winattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p],
+    "ssd_winattn_store_rope": [c_void_p, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_moe_route_sigmoid_grouped": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_gemm_rows_glu_clamp": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p],
+    "ssd_embed_hist": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_void_p],
+    "ssd_postnorm_tail": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_long, c_int, c_void_p,
+                          c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_rmsnorm_w32_rows": [c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_rope_rows": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int, c_void_p],
+    "ssd_gate_rows": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_token_shift_mix": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
                             c_int, c_void_p],
     "ssd_wkv_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -180,6 +190,8 @@ FAMILY_SOURCES = {
     "fatulix": _COMMON_ROWS + ["attention_diff.hip"],
     "zerusun": _COMMON_ROWS + ["dyt.hip", "attention_latent.hip", "lightning.hip"],
     "fomunex": _COMMON_ROWS + ["prenorm.hip", "attention_window.hip", "recurrent.hip"],
+    "dosuvik": _COMMON_ROWS + ["postnorm.hip", "prenorm.hip", "attention_window.hip", "attention_latent.hip", "lightning.hip",
+                               "recurrent.hip"],
 }
 
 

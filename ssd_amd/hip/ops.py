@@ -505,10 +505,14 @@ def latent_attn_mfma_ok(kv_rank: int, rot: int, f32: bool) -> bool:
     return load_library().ssd_latent_attn_mfma_ok(kv_rank, rot, int(f32)) == 1
 
 
+SCAN_SILU, SCAN_RAW = 0, 1
+
+
 def lightning_scan(proj, ld: int, q_off: int, k_off: int, v_off: int, decay, positions, state_slots, state, out_rows, B: int, H: int,
-                   D: int, Dv: int, cu_q=None, q_per_seq: int = 0):
+                   D: int, Dv: int, cu_q=None, q_per_seq: int = 0, act: int = SCAN_SILU):
+    """act SCAN_SILU: q, k, v = silu of the row's values; SCAN_RAW: the values as they are (the caller prepared them)."""
     _check(load_library().ssd_lightning_scan(_p(proj), ld, q_off, k_off, v_off, _p(decay), _p(positions), _p(cu_q), q_per_seq,
-                                             _p(state_slots), _p(state), _p(out_rows), B, H, D, Dv, _stream()), "ssd_lightning_scan")
+                                             _p(state_slots), _p(state), _p(out_rows), B, H, D, Dv, act, _stream()), "ssd_lightning_scan")
 
 
 def lightning_gate_norm(o_rows, proj, ld: int, g_off: int, weight, eps: float, out_rows, T: int, N: int, f32: bool):
@@ -571,11 +575,19 @@ def winattn_store(qkv, ld: int, eps: float, slots, q_out, k_cache, v_cache, T: i
 
 def winattn_paged(q, k_cache, v_cache, slopes, sinks, block_tables, max_blocks: int, positions, B: int, T: int, H: int, G: int, D: int,
                   Dv: int, block_size: int, window: int, scale: float, cap: float, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0,
-                  max_q: int = 0):
-    """max_q > 0 (an upper bound of the rows a sequence brings; bf16, aligned head sizes, block_size % 32 == 0): the MFMA form."""
+                  max_q: int = 0, out_freqs=None):
+    """max_q > 0 (an upper bound of the rows a sequence brings; bf16, aligned head sizes, block_size % 32 == 0): the MFMA form.
+    out_freqs (fp32 [Dv / 2]): every head's output turns back by the query's position (values cached rotated by their own)."""
     _check(load_library().ssd_winattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(slopes), _p(sinks), _p(block_tables), max_blocks,
                                             _p(positions), _p(cu_q), q_per_seq, max_q, B, T, H, G, D, Dv, block_size, window, scale, cap,
-                                            _p(out_rows), int(f32), _stream()), "ssd_winattn_paged")
+                                            _p(out_freqs), _p(out_rows), int(f32), _stream()), "ssd_winattn_paged")
+
+
+def winattn_store_rope(qkv, ld: int, q_norm_w, k_norm_w, eps: float, positions, qk_freqs, rot_dims: int, v_freqs, slots, q_out, k_cache,
+                       v_cache, T: int, H: int, G: int, D: int, Dv: int, block_size: int, f32: bool):
+    _check(load_library().ssd_winattn_store_rope(_p(qkv), ld, _p(q_norm_w), _p(k_norm_w), eps, _p(positions), _p(qk_freqs), rot_dims,
+                                                 _p(v_freqs), _p(slots), _p(q_out), _p(k_cache), _p(v_cache), T, H, G, D, Dv, block_size,
+                                                 int(f32), _stream()), "ssd_winattn_store_rope")
 
 
 def token_shift_mix(hn, mu, shift_state, positions, state_slots, B: int, out_rows, T: int, W: int, S: int, f32: bool, cu_q=None,
@@ -609,3 +621,44 @@ def ssd_scan(xbc, ldx: int, x_off: int, b_off: int, c_off: int, proj, ld: int, d
 def group_gate_norm(o_rows, gate_rows, ldg: int, weight, eps: float, out_rows, T: int, N: int, groups: int, gate_first: bool, f32: bool):
     _check(load_library().ssd_group_gate_norm(_p(o_rows), _p(gate_rows), ldg, _p(weight), eps, _p(out_rows), T, N, groups,
                                               int(gate_first), int(f32), _stream()), "ssd_group_gate_norm")
+
+
+# ---- layers that normalise a sublayer's output only, depth-weighted average, retention, grouped sigmoid router ----
+
+def embed_hist(ids, table, x_out, T: int, W: int, f32: bool, hist0=None, rows_out=None):
+    _check(load_library().ssd_embed_hist(_p(ids), _p(table), _p(x_out), _p(hist0), _p(rows_out), T, W, table.shape[0], int(f32), _stream()),
+           "ssd_embed_hist")
+
+
+def postnorm_tail(x, post_weight, eps: float, T: int, W: int, f32: bool, *, y=None, ydn=None, inv=None, weights=None, top: int = 0,
+                  hist=None, hist_stride: int = 0, hist_levels: int = 0, coef=None, next_out=None):
+    """x += post_weight * rms(y | routed mix of ydn); hist: level hist_levels - 1 = x, then x = sum_j coef[j] * level_j; next_out = x
+    as element-type rows."""
+    _check(load_library().ssd_postnorm_tail(_p(y), _p(ydn), _p(inv), _p(weights), top, _p(post_weight), eps, _p(x), _p(hist), hist_stride,
+                                            hist_levels, _p(coef), _p(next_out), T, W, int(f32), _stream()), "ssd_postnorm_tail")
+
+
+def rmsnorm_w32_rows(x, weight, eps: float, out_rows, T: int, W: int, f32: bool, gather=None):
+    _check(load_library().ssd_rmsnorm_w32_rows(_p(x), _p(weight), eps, _p(out_rows), _p(gather), T, W, int(f32), _stream()),
+           "ssd_rmsnorm_w32_rows")
+
+
+def rope_rows(rows, ld: int, positions, freqs, rot_dims: int, heads: int, D: int, T: int, off_a: int, scale_a: float = 1.0,
+              off_b: int = -1, scale_b: float = 1.0):
+    _check(load_library().ssd_rope_rows(_p(rows), ld, _p(positions), _p(freqs), rot_dims, heads, D, off_a, scale_a, off_b, scale_b, T,
+                                        _stream()), "ssd_rope_rows")
+
+
+def gate_rows(o_rows, ldo: int, gate_rows_, ldg: int, out_rows, T: int, N: int, f32: bool):
+    _check(load_library().ssd_gate_rows(_p(o_rows), ldo, _p(gate_rows_), ldg, _p(out_rows), T, N, int(f32), _stream()), "ssd_gate_rows")
+
+
+def moe_route_sigmoid_grouped(logits, ld: int, correction, idx, weights, T: int, E: int, top: int, groups: int, keep: int,
+                              group_top: int = 2):
+    _check(load_library().ssd_moe_route_sigmoid_grouped(_p(logits), ld, _p(correction), _p(idx), _p(weights), T, E, top, groups, keep,
+                                                        group_top, _stream()), "ssd_moe_route_sigmoid_grouped")
+
+
+def gemm_rows_glu_clamp(x, w, y, M: int, N: int, K: int, limit: float, alpha: float):
+    """Dense product with the clamped swish-GLU as epilogue (bf16; weight rows in (gate, up) pairs): y [M][N / 2]."""
+    _check(load_library().ssd_gemm_rows_glu_clamp(_p(x), _p(w), _p(y), M, N, K, limit, alpha, _stream()), "ssd_gemm_rows_glu_clamp")

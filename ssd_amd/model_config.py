@@ -526,8 +526,181 @@ class FomunexConfig:
                              float(cfg.get("logit_scale") or 1.0), float(cfg.get("logit_softcap") or 0.0))
 
 
+# --------------------------------------------------------------------------------------------------
+# Dosuvik: layers that normalise a sublayer's OUTPUT only (x <- x + (1 + w) rms(f(x))) over an fp32 residual, followed by a learned
+# weighted average over the results of all earlier layers; mixers are retention (linear attention with a fixed decay and rotary
+# positions), gated latent attention, or windowed grouped-query attention with rotated values and a sink; feed-forwards are a dense
+# clamped swish-GLU or sigmoid-routed silu-GLU experts with a choice correction and group-limited choice
+# --------------------------------------------------------------------------------------------------
+@dataclass
+class Rotary:
+    """Rotary positions on the first `dims` entries of a head: pair i turns by position * base^(-2i/dims).  layout "halves" pairs
+    entry i with i + dims / 2, "interleaved" pairs entry 2i with 2i + 1."""
+    dims: int
+    base: float
+    layout: str = "halves"
+
+    def frequencies(self, dims: int | None = None) -> list[float]:
+        d = self.dims if dims is None else dims
+        return [self.base ** (-2.0 * i / d) for i in range(d // 2)]
+
+    def to_halves(self, width: int) -> list[int]:
+        """The order of a `width`-wide rotated part that turns this layout into the "halves" layout (the identity for "halves"): a dot
+        product of two parts permuted alike is unchanged, so weights whose output rows are permuted so serve kernels that pair i with
+        i + dims / 2."""
+        if self.layout == "halves":
+            return list(range(width))
+        return list(range(0, self.dims, 2)) + list(range(1, self.dims, 2)) + list(range(self.dims, width))
+
+
+@dataclass
+class RetentionMixer:
+    """Linear attention with one fixed decay per head and no softmax: rotary q and k, k scaled by dim^-0.5 after the rotation, per head
+    S <- decay S + k v^T and o = S^T q over a recurrent fp32 [dim][vdim] state; each head's o divided by its root mean square (no
+    weight), times silu(W_g h), projected."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: list
+    rope: Rotary
+    kind: str = "retention"
+
+
+@dataclass
+class GatedLatentAttention:
+    """Attention whose keys and values come from a cached low-rank latent (kv_rank wide, RMS-normed) plus ONE rotated key part shared by
+    all heads; queries straight from the hidden row, per head `dim` unrotated + `rot_dim` rotated entries; ordinary causal softmax
+    (window 0 = every earlier token); the concatenated heads times sigmoid(W_g h) element by element."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    rope: Rotary
+    window: int = 0
+    kind: str = "latent_attention"
+
+
+@dataclass
+class RotaryWindowAttention:
+    """Grouped-query attention with an RMS norm (plain weights) over the WHOLE q and the whole k projection before the heads are split,
+    rotary q / k on the first rope.dims entries, values rotated by their own position over all vdim entries (cached so) and every
+    head's output turned back by the query's position, a sliding window (0 = every earlier token) and a learned per-head sink in the
+    softmax denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+    rope: Rotary
+    rotate_values: bool = True
+    kind: str = "attention"
+
+
+@dataclass
+class ClampedGluMLP:
+    """Dense feed-forward W_down(g sigmoid(1.702 g) (u + 1)), g = min(W_gate h, limit), u = clamp(W_up h, +-limit)."""
+    ff: int
+    limit: float
+    kind: str = "dense"
+
+
+@dataclass
+class BiasedGroupRoutedMLP:
+    """Mixture of silu-GLU experts behind a sigmoid router: scores s = sigmoid(W_r h); the choice uses s + correction, the weights use
+    s as it is; experts in `groups` contiguous groups, a group's score = the sum of its two largest choice scores, only experts of the
+    best `keep` groups can be chosen; the `top` largest choice scores win; weights are not renormalised."""
+    experts: int
+    top: int
+    ff: int
+    groups: int = 1
+    keep: int = 1
+    kind: str = "moe"
+
+
+@dataclass
+class DosuvikLayer:
+    mixer: object               # RetentionMixer | GatedLatentAttention | RotaryWindowAttention
+    mlp: object                 # ClampedGluMLP | BiasedGroupRoutedMLP | None
+
+
+@dataclass
+class DosuvikConfig:
+    """config.json keys: architecture, vocab, width, norm.eps, layers[{type, mixer{...}, mlp{kind, ...} | null}]."""
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float
+    layers: list = field(default_factory=list)
+    family: str = "dosuvik"
+    max_position_embeddings: int = 1 << 20
+    tie_word_embeddings: bool = False
+
+    SWISH_ALPHA = 1.702         # the dense feed-forward's gate is g * sigmoid(1.702 g)
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def recurrent(self) -> bool:
+        """True when some layer keeps a per-sequence state that is not a function of cached pages."""
+        return any(l.mixer.kind == "retention" for l in self.layers)
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+    @staticmethod
+    def from_json(cfg: dict) -> "DosuvikConfig":
+        layers = []
+        for lc in cfg["layers"]:
+            m, kind = lc["mixer"], lc["type"]
+            r = m["rot"]
+            if kind == "retention":
+                mixer = RetentionMixer(int(m["heads"]), int(m["dim"]), int(m["vdim"]), [float(d) for d in m["decay"]],
+                                       Rotary(int(r["dims"]), float(r["base"]), "halves"))
+                if len(mixer.decay) != mixer.heads:
+                    raise ValueError("Dosuvik: one decay per head")
+                width = mixer.dim
+            elif kind == "latent_attention":
+                mask = m.get("mask") or {}
+                mixer = GatedLatentAttention(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                                             float(m["scale"]), Rotary(int(r["dims"]), float(r["base"]), "interleaved"),
+                                             int(mask.get("size") or 0))
+                width = mixer.rot_dim
+            elif kind == "attention":
+                mask = m.get("mask") or {}
+                mixer = RotaryWindowAttention(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]),
+                                              int(mask.get("size") or 0), Rotary(int(r["dims"]), float(r["base"]), "halves"))
+                if mixer.heads % mixer.kv_heads or mixer.vdim % 2:
+                    raise ValueError("Dosuvik: heads must be a multiple of kv_heads and vdim even")
+                width = mixer.dim
+            else:
+                raise ValueError(f"Dosuvik: unknown layer type {kind!r}")
+            if mixer.rope.dims % 2 or not 0 <= mixer.rope.dims <= width:
+                raise ValueError("Dosuvik: rot.dims must be even and at most the rotated part's size")
+            ml = lc.get("mlp")
+            mlp = None
+            if ml is not None:
+                if ml["kind"] == "dense":
+                    mlp = ClampedGluMLP(int(ml["ff"]), float(ml["limit"]))
+                elif ml["kind"] == "moe":
+                    rt = ml["router"]
+                    g = rt.get("groups") or {}
+                    mlp = BiasedGroupRoutedMLP(int(rt["experts"]), int(rt["top"]), int(ml["expert"]["ff"]), int(g.get("count", 1)),
+                                               int(g.get("keep", g.get("count", 1))))
+                    if mlp.experts % mlp.groups or not (1 <= mlp.keep <= mlp.groups) or not (1 <= mlp.top <= mlp.experts // mlp.groups * mlp.keep):
+                        raise ValueError("Dosuvik: router groups do not fit the experts")
+                else:
+                    raise ValueError(f"Dosuvik: unknown feed-forward kind {ml['kind']!r}")
+            layers.append(DosuvikLayer(mixer, mlp))
+        return DosuvikConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers)
+
+
 # config.json "architecture" values that are read by this package's own readers (everything else goes through transformers' AutoConfig)
-ARCHITECTURES = {"Fatulix": FatulixConfig.from_json, "Zerusun": ZerusunConfig.from_json, "Fomunex": FomunexConfig.from_json}
+ARCHITECTURES = {"Fatulix": FatulixConfig.from_json, "Zerusun": ZerusunConfig.from_json, "Fomunex": FomunexConfig.from_json,
+                 "Dosuvik": DosuvikConfig.from_json}
 
 
 def read_native_config(model_dir: str):

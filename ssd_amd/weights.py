@@ -138,6 +138,36 @@ def fomunex_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
     return out + [("final.norm", ()), ("head", (cfg.vocab_size, W))]
 
 
+def dosuvik_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
+    """Tensor names and shapes of a Dosuvik checkpoint (model_config.DosuvikConfig).  Layer i ends with 'l<i>.dwa', the i + 2 weights
+    of the average over the embedding output and the results of layers 0 .. i."""
+    W = cfg.hidden_size
+    out = [("embed", (cfg.vocab_size, W))]
+    for i, lc in enumerate(cfg.layers):
+        p, m, ml = f"l{i}.", lc.mixer, lc.mlp
+        out += [(p + "norm1", (W,))] + ([(p + "norm2", (W,))] if ml is not None else [])
+        if m.kind == "retention":
+            n, nv = m.heads * m.dim, m.heads * m.vdim
+            out += [(p + "mix.q", (n, W)), (p + "mix.k", (n, W)), (p + "mix.v", (nv, W)), (p + "mix.g", (nv, W)), (p + "mix.o", (W, nv))]
+        elif m.kind == "latent_attention":
+            nv = m.heads * m.vdim
+            out += [(p + "mix.q", (m.heads * (m.dim + m.rot_dim), W)), (p + "mix.dkv", (m.kv_rank + m.rot_dim, W)),
+                    (p + "mix.dkv.norm", (m.kv_rank,)), (p + "mix.uk", (m.heads * m.dim, m.kv_rank)), (p + "mix.uv", (nv, m.kv_rank)),
+                    (p + "mix.g", (nv, W)), (p + "mix.o", (W, nv))]
+        else:
+            out += [(p + "mix.q", (m.heads * m.dim, W)), (p + "mix.k", (m.kv_heads * m.dim, W)), (p + "mix.v", (m.kv_heads * m.vdim, W)),
+                    (p + "mix.q.norm", (m.heads * m.dim,)), (p + "mix.k.norm", (m.kv_heads * m.dim,)), (p + "mix.sink", (m.heads,)),
+                    (p + "mix.o", (W, m.heads * m.vdim))]
+        if ml is not None and ml.kind == "dense":
+            out += [(p + "mlp.gate", (ml.ff, W)), (p + "mlp.up", (ml.ff, W)), (p + "mlp.down", (W, ml.ff))]
+        elif ml is not None:
+            for e in range(ml.experts):
+                out += [(p + f"mlp.e{e}.gate", (ml.ff, W)), (p + f"mlp.e{e}.up", (ml.ff, W)), (p + f"mlp.e{e}.down", (W, ml.ff))]
+            out += [(p + "mlp.router", (ml.experts, W)), (p + "mlp.correction", (ml.experts,))]
+        out.append((p + "dwa", (i + 2,)))
+    return out + [("final.norm", (W,)), ("head", (cfg.vocab_size, W))]
+
+
 def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
     if cfg.family == "eagle3":
         return eagle_param_shapes(cfg)
@@ -147,6 +177,8 @@ def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
         return zerusun_param_shapes(cfg)
     if cfg.family == "fomunex":
         return fomunex_param_shapes(cfg)
+    if cfg.family == "dosuvik":
+        return dosuvik_param_shapes(cfg)
     h, hd, nh, nkv, I, V = cfg.hidden_size, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, cfg.intermediate_size, cfg.vocab_size
     out = [("model.embed_tokens.weight", (V, h))]
     for i in range(cfg.num_layers):
@@ -408,6 +440,11 @@ def synthetic_weights(cfg: ModelConfig, seed: int, std: float, rank: int = 0, tp
         recipe = dict(recipe, family=cfg.family)
     for name, shape in param_shapes(cfg):
         w = shard_param(cfg, name, synthetic_tensor(name, shape, seed, std, gen_device, norm_jitter, recipe), rank, tp)
+        if cfg.family == "dosuvik":
+            if name.endswith((".norm1", ".norm2")) or name == "final.norm":       # stored around zero: the norm multiplies by 1 + w
+                w = (w.float() - 1.0).to(w.dtype)
+            elif name.endswith(".dwa"):         # mostly the newest result, a little of every earlier one
+                w = (w.float() * 0.1 + torch.nn.functional.one_hot(torch.tensor(shape[0] - 1), shape[0]).to(w.device)).to(w.dtype)
         yield name, (w.to(out_device) if out_device is not None else w)
 
 
