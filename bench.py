@@ -69,11 +69,11 @@ def parse(argv=None):
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c2", "c5t", "c4e", "tiny", "tiny-async", "tiny-eagle", "fatulix", "zerusun", "fomunex"])
-    ap.add_argument("--arch-size", default="all", help="--workload fatulix | zerusun | fomunex: one of the sizes in ssd_amd/utils/arch_bench.py SIZES, or all")
-    ap.add_argument("--arch-batch", type=int, default=0, help="--workload fatulix | zerusun | fomunex: decode batch (0 = 1 and 8)")
-    ap.add_argument("--arch-only", default="both", choices=["both", "fatulix", "llama", "zerusun", "fomunex"],
-                    help="--workload fatulix | zerusun | fomunex: which family of the pair to run")
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c2", "c5t", "c4e", "tiny", "tiny-async", "tiny-eagle", "fatulix", "zerusun", "fomunex", "dosuvik"])
+    ap.add_argument("--arch-size", default="all", help="--workload fatulix | zerusun | fomunex | dosuvik: one of the sizes in ssd_amd/utils/arch_bench.py SIZES, or all")
+    ap.add_argument("--arch-batch", type=int, default=0, help="--workload fatulix | zerusun | fomunex | dosuvik: decode batch (0 = 1 and 8)")
+    ap.add_argument("--arch-only", default="both", choices=["both", "fatulix", "llama", "zerusun", "fomunex", "dosuvik"],
+                    help="--workload fatulix | zerusun | fomunex | dosuvik: which family of the pair to run")
     ap.add_argument("--k", type=int, default=None, help="speculation length (default: 7 async, 6 sync)")
     ap.add_argument("--f", type=int, default=3, help="async fan-out")
     ap.add_argument("--placement", default="auto", choices=["auto", "colocated", "dedicated"])
@@ -440,6 +440,10 @@ def main():
     if args.workload == "fomunex":      # the Fomunex decoder beside an equal-size Zerusun decoder; single GPU
         from ssd_amd.utils.arch_bench import run_fomunex
         print(json.dumps(run_fomunex(args)), flush=True)
+        return
+    if args.workload == "dosuvik":      # the Dosuvik decoder beside an equal-size Zerusun decoder; single GPU
+        from ssd_amd.utils.arch_bench import run_dosuvik
+        print(json.dumps(run_dosuvik(args)), flush=True)
         return
     if args.workload == "zerusun":      # the Zerusun decoder beside an equal-size Fatulix decoder; single GPU
         from ssd_amd.utils.arch_bench import run_zerusun

@@ -13,7 +13,11 @@ token (three-matrix experts of 2/3 the two-matrix experts' ff), mixers of about 
 space; sigmoid-routed clamped-GLU experts and one PolyNorm dense feed-forward) beside the closest existing family, Zerusun (fp32
 residual, a windowed attention over a paged cache next to a recurrent mixer over state slots, routed three-matrix experts), at equal
 size: the same width, layers, vocabulary, experts, top and active feed-forward parameters per token, the same window, mixers of about
-the same parameter count."""
+the same parameter count.
+--workload dosuvik: the Dosuvik decoder (output-norm layers with a depth average; latent attention / retention / windowed attention with
+rotated values and a sink / retention; grouped sigmoid-routed silu-GLU experts and one dense clamped GLU) beside the closest existing
+family, Zerusun (the same latent attention and linear-attention scan kernels, a grouped router, silu-GLU experts), at equal size.
+"""
 from __future__ import annotations
 
 import json
@@ -24,6 +28,8 @@ import torch
 from ssd_amd.config import Config
 from ssd_amd.engine.block_manager import BlockManager
 from ssd_amd.engine.sequence import Sequence
+from ssd_amd.model_config import (BiasedGroupRoutedMLP, ClampedGluMLP, DosuvikConfig, DosuvikLayer, GatedLatentAttention, RetentionMixer,
+                                  Rotary, RotaryWindowAttention)
 from ssd_amd.model_config import (DiffAttention, FatulixConfig, FatulixLayer, FomunexConfig, FomunexLayer, GroupRoutedMLP, LatentAttention,
                                   LightningAttention, Mamba2Mixer, ModelConfig, PolyNormMLP, RopeSpec, RoutedMLP, SigmoidRoutedMLP,
                                   WindowAttention, WkvMixer, ZerusunConfig, ZerusunLayer)
@@ -71,6 +77,22 @@ def fomunex_models(size: str):
     for i, l in enumerate(fom.layers):
         fom.layers[i] = FomunexLayer(l.mixer, l.mlp, i)
     return fom, zer
+
+
+def dosuvik_models(size: str):
+    """(Dosuvik, Zerusun) of equal size: the same width, layers, vocabulary, experts, top, router groups, latent and state sizes; the
+    experts carry what Zerusun's experts and its shared expert carry per token together, one layer has the dense feed-forward of the
+    same active parameter count."""
+    W, L, Hh, G, E, top, ff, sff, inter = SIZES[size]
+    zer, _ = zerusun_models(size)
+    ffx = (ff + sff // top) * 2 // 3
+    moe = BiasedGroupRoutedMLP(E, top, ffx, 4, 2)
+    dense = ClampedGluMLP(top * ffx, 7.0)
+    lat = GatedLatentAttention(Hh, 128, 64, 128, 512, 192 ** -0.5, Rotary(64, 1e6, "interleaved"), 1024)
+    ret = RetentionMixer(Hh // 2, 128, 128, [1.0 - 2.0 ** -(3 + 5 * h / (Hh // 2)) for h in range(Hh // 2)], Rotary(128, 1e6))
+    att = RotaryWindowAttention(Hh, G, 128, 128, 128 ** -0.5, 1024, Rotary(64, 1e4))
+    layers = [DosuvikLayer(lat, moe), DosuvikLayer(ret, dense), DosuvikLayer(att, moe), DosuvikLayer(ret, moe)]
+    return DosuvikConfig(VOCAB, W, 1e-5, (layers * (L // 4 + 1))[:L]), zer
 
 
 def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
@@ -170,6 +192,36 @@ def run_zerusun(args) -> dict:
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights, random tokens)",
             "config": {"model": "zerusun-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
             "closest_model_value": results[k]["fatulix_equal_size"]["decode_tok_s"], "sizes": results}
+
+
+def run_dosuvik(args) -> dict:
+    """bench.py --workload dosuvik: the Dosuvik decoder beside an equal-size Zerusun decoder (the family that shares its latent
+    attention, its linear-attention scan, its grouped router and its silu-GLU experts)."""
+    sizes = list(SIZES) if args.arch_size == "all" else [args.arch_size]
+    batches = [args.arch_batch] if args.arch_batch else [1, 8]
+    only = getattr(args, "arch_only", "both")
+    prompt_len, steps, warmup = 2048, max(args.steps, 8), max(args.warmup, 2)
+    results = {}
+    for size in sizes:
+        dos, zer = dosuvik_models(size)
+        for b in batches:
+            key = f"{size}_b{b}"
+            results[key] = {}
+            if only in ("both", "dosuvik"):
+                results[key]["dosuvik"] = measure(dos, prompt_len, b, steps, warmup)
+            if only in ("both", "zerusun"):
+                results[key]["zerusun_equal_size"] = measure(zer, prompt_len, b, steps, warmup)
+            print(f"[arch_bench] {key}: {json.dumps(results[key])}", flush=True)
+    k = "w4096_b8"
+    if k not in results or len(results[k]) < 2:
+        return {"metric": "Dosuvik / equal-size Zerusun throughput (partial run)", "sizes": results}
+    return {"metric": "decode tokens/s, Dosuvik w4096 (4 layers: latent attention / retention / windowed attention / retention, 16 "
+                      "experts top 2), batch 8, beside an equal-size Zerusun decoder",
+            "value": results[k]["dosuvik"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": results[k]["dosuvik"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"model": "dosuvik-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
+            "closest_model_value": results[k]["zerusun_equal_size"]["decode_tok_s"], "sizes": results}
 
 
 def run_fomunex(args) -> dict:
