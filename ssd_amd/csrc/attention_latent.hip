@@ -53,6 +53,7 @@ __device__ __forceinline__ float rope_entry(F x, int i, int R, int rot_dims, flo
   return i < half ? x(i) * c - x(i + half) * s : x(i) * c + x(i - half) * s;
 }
 
+// grid = (tokens, column blocks): every workgroup of a token computes the row's statistics itself and takes a share of the columns.
 template <typename T>
 __global__ void __launch_bounds__(256)
 latent_store_kernel(const float* __restrict__ proj, long ld, int Qr, int Cr, int R, int H, const T* __restrict__ wq,
@@ -61,29 +62,31 @@ latent_store_kernel(const float* __restrict__ proj, long ld, int Qr, int Cr, int
                     float* __restrict__ gate_out) {
   __shared__ float red[4];
   const size_t t = blockIdx.x;
+  const int first = blockIdx.y * 256 + threadIdx.x, step = 256 * gridDim.y;
   const float* pr = proj + t * ld;
   const float* dq = pr;
   const float* dkv = pr + Qr;
   float sq = 0.f, sc = 0.f;
-  for (int i = threadIdx.x; i < Qr; i += 256) sq += dq[i] * dq[i];
+  if (wq)
+    for (int i = threadIdx.x; i < Qr; i += 256) sq += dq[i] * dq[i];
   for (int i = threadIdx.x; i < Cr; i += 256) sc += dkv[i] * dkv[i];
-  sq = block_sum_256(sq, red);
+  if (wq) sq = block_sum_256(sq, red);
   sc = block_sum_256(sc, red);
   const float rq = 1.0f / sqrtf(sq / (float)Qr + eps), rc = 1.0f / sqrtf(sc / (float)Cr + eps);
   if (wq) {
-    for (int i = threadIdx.x; i < Qr; i += 256) stf<T>(cq_out + t * Qr + i, dq[i] * rq * ldf<T>(wq + i));
+    for (int i = first; i < Qr; i += step) stf<T>(cq_out + t * Qr + i, dq[i] * rq * ldf<T>(wq + i));
   } else {                                            // queries that pass through no latent: the first Qr entries as they are
-    for (int i = threadIdx.x; i < Qr; i += 256) stf<T>(cq_out + t * Qr + i, dq[i]);
+    for (int i = first; i < Qr; i += step) stf<T>(cq_out + t * Qr + i, dq[i]);
   }
   if (gate_out)
-    for (int i = threadIdx.x; i < H; i += 256) gate_out[t * H + i] = sigmoidf_(pr[Qr + Cr + R + i]);
+    for (int i = first; i < H; i += step) gate_out[t * H + i] = sigmoidf_(pr[Qr + Cr + R + i]);
   const int slot = slots[t];
   if (slot < 0) return;
   T* row = cache + (size_t)slot * (Cr + R);
-  for (int i = threadIdx.x; i < Cr; i += 256) stf<T>(row + i, dkv[i] * rc * ldf<T>(wkv + i));
+  for (int i = first; i < Cr; i += step) stf<T>(row + i, dkv[i] * rc * ldf<T>(wkv + i));
   const float pos = (float)positions[t];
   const float* kr = dkv + Cr;
-  for (int i = threadIdx.x; i < R; i += 256)
+  for (int i = first; i < R; i += step)
     stf<T>(row + Cr + i, rope_entry([&](int j) { return kr[j]; }, i, R, rot_dims, pos, freqs, mag));
 }
 
@@ -381,12 +384,14 @@ extern "C" int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int 
   if (T <= 0 || q_rank <= 0 || kv_rank <= 0 || rot < 0 || H <= 0 || rot_dims < 0 || rot_dims > rot || (rot_dims & 1) ||
       ld < (long)q_rank + kv_rank + rot + (gate_out ? H : 0))
     return SSD_ERR_SHAPE;
+  const int cols = q_rank > kv_rank ? q_rank : kv_rank;
+  const dim3 grid(T, T >= 64 ? 1 : ((cols + 255) / 256 < 16 ? (cols + 255) / 256 : 16));
   if (f32)
-    hipLaunchKernelGGL(latent_store_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_rank,
+    hipLaunchKernelGGL(latent_store_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_rank,
                        kv_rank, rot, H, (const float*)q_norm_w, (const float*)kv_norm_w, eps, positions, freqs, mag, rot_dims, slots,
                        (float*)cq_out, (float*)cache, (float*)gate_out);
   else
-    hipLaunchKernelGGL(latent_store_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_rank,
+    hipLaunchKernelGGL(latent_store_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_rank,
                        kv_rank, rot, H, (const bf16_t*)q_norm_w, (const bf16_t*)kv_norm_w, eps, positions, freqs, mag, rot_dims, slots,
                        (bf16_t*)cq_out, (bf16_t*)cache, (float*)gate_out);
   return LAUNCH_OK();

@@ -75,8 +75,10 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-// One workgroup per token.  q' = w_q * q / rms(q) over all H * D entries (k alike over G * D), then per head the pair (i, i + half)
-// turns by pos * qk_freqs[i]; v heads turn over all Dv entries by pos * v_freqs[i] (v_freqs NULL: stored as they are).
+// q' = w_q * q / rms(q) over all H * D entries (k alike over G * D), then per head the pair (i, i + half) turns by pos * qk_freqs[i];
+// v heads turn over all Dv entries by pos * v_freqs[i] (v_freqs NULL: stored as they are).  grid = (tokens, column blocks): every
+// workgroup of a token sums the squares of the whole row itself (a few thousand cached floats) and takes a share of the work items --
+// a pair that turns (one sine and cosine for both entries) or a single entry that does not.
 template <typename T>
 __global__ void __launch_bounds__(256)
 winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __restrict__ wq, const T* __restrict__ wk, float eps,
@@ -85,7 +87,7 @@ winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __res
                           T* __restrict__ kc, T* __restrict__ vc, int H, int G, int D, int Dv, int bs) {
   __shared__ float red[4];
   const int t = blockIdx.x;
-  const int Nq = H * D, Nk = G * D, Nv = G * Dv;
+  const int Nq = H * D, Nk = G * D;
   const float* row = qkv + (size_t)t * ld;
   const float pos = (float)positions[t];
   const int slot = slots[t];
@@ -97,38 +99,41 @@ winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __res
   sq = block_sum_256(sq, red);
   sk = block_sum_256(sk, red);
   const float rq = 1.0f / sqrtf(sq / (float)Nq + eps), rk = 1.0f / sqrtf(sk / (float)Nk + eps);
-  const int half = rot_dims >> 1;
-  for (int i = threadIdx.x; i < Nq + Nk; i += 256) {
-    const bool isq = i < Nq;
-    const int j = isq ? i : i - Nq, d = j % D;
-    const float* src = row + (isq ? 0 : Nq);
-    const T* w = isq ? wq : wk;
-    const float r = isq ? rq : rk;
-    float v = src[j] * r * ldf<T>(w + j);
-    if (d < rot_dims) {
-      const int f = d < half ? d : d - half;
-      const int jp = d < half ? j + half : j - half;
-      const float o = src[jp] * r * ldf<T>(w + jp);
-      const float ang = pos * qk_freqs[f];
-      const float c = cosf(ang), sn = sinf(ang);
-      v = d < half ? v * c - o * sn : v * c + o * sn;
+  const int half = rot_dims >> 1, per = D - half;          // items of a q / k head: `half` pairs, then the entries that do not turn
+  const int hv = Dv >> 1, perv = v_freqs ? hv : Dv;        // items of a v head
+  const int n_qk = (H + G) * per, n_all = n_qk + (slot >= 0 ? G * perv : 0);
+  for (int u = blockIdx.y * 256 + threadIdx.x; u < n_all; u += 256 * gridDim.y) {
+    if (u < n_qk) {
+      const int hd = u / per, i = u % per;
+      const bool isq = hd < H;
+      if (!isq && slot < 0) continue;
+      const int base = hd * D;                             // k heads follow the q heads in the row, and their weights in wk
+      const T* w = isq ? wq + base : wk + (base - Nq);
+      const float r = isq ? rq : rk;
+      T* dst = isq ? q_out + (size_t)t * Nq + base : kc + (((size_t)blk * G + (hd - H)) * bs + off) * D;
+      if (i < half) {
+        const float a = row[base + i] * r * ldf<T>(w + i), b = row[base + i + half] * r * ldf<T>(w + i + half);
+        float sn, c;
+        sincosf(pos * qk_freqs[i], &sn, &c);
+        stf<T>(dst + i, a * c - b * sn);
+        stf<T>(dst + i + half, b * c + a * sn);
+      } else {
+        stf<T>(dst + i + half, row[base + i + half] * r * ldf<T>(w + i + half));
+      }
+    } else {
+      const int g = (u - n_qk) / perv, i = (u - n_qk) % perv;
+      const float* src = row + Nq + Nk + g * Dv;
+      T* dst = vc + (((size_t)blk * G + g) * Dv) * bs + off;
+      if (v_freqs) {
+        const float a = src[i], b = src[i + hv];
+        float sn, c;
+        sincosf(pos * v_freqs[i], &sn, &c);
+        stf<T>(dst + (size_t)i * bs, a * c - b * sn);
+        stf<T>(dst + (size_t)(i + hv) * bs, b * c + a * sn);
+      } else {
+        stf<T>(dst + (size_t)i * bs, src[i]);
+      }
     }
-    if (isq) stf<T>(q_out + (size_t)t * Nq + j, v);
-    else if (slot >= 0) stf<T>(kc + (((size_t)blk * G + j / D) * bs + off) * D + d, v);
-  }
-  if (slot < 0) return;
-  const int hv = Dv >> 1;
-  for (int cI = threadIdx.x; cI < Nv; cI += 256) {
-    const int g = cI / Dv, d = cI % Dv;
-    float v = row[Nq + Nk + cI];
-    if (v_freqs) {
-      const int f = d < hv ? d : d - hv;
-      const float o = row[Nq + Nk + (d < hv ? cI + hv : cI - hv)];
-      const float ang = pos * v_freqs[f];
-      const float c = cosf(ang), sn = sinf(ang);
-      v = d < hv ? v * c - o * sn : v * c + o * sn;
-    }
-    stf<T>(vc + (((size_t)blk * G + g) * Dv + d) * bs + off, v);
   }
 }
 
@@ -497,12 +502,15 @@ extern "C" int ssd_winattn_store_rope(const void* qkv_rows, long ld, const void*
   if (T <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || block_size <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1) ||
       (v_freqs && (Dv & 1)) || ld < (long)(H + G) * D + (long)G * Dv)
     return SSD_ERR_SHAPE;
+  const int items = (H + G) * (D - rot_dims / 2) + G * (v_freqs ? Dv / 2 : Dv);
+  const int yb = T >= 64 ? 1 : ((items + 255) / 256 < 16 ? (items + 255) / 256 : 16);
+  const dim3 grid(T, yb);
   if (f32)
-    hipLaunchKernelGGL(winattn_store_rope_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
+    hipLaunchKernelGGL(winattn_store_rope_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
                        (const float*)q_norm_w, (const float*)k_norm_w, eps, positions, qk_freqs, rot_dims, v_freqs, slots,
                        (float*)q_out, (float*)k_cache, (float*)v_cache, H, G, D, Dv, block_size);
   else
-    hipLaunchKernelGGL(winattn_store_rope_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
+    hipLaunchKernelGGL(winattn_store_rope_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)qkv_rows, ld,
                        (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, positions, qk_freqs, rot_dims, v_freqs, slots,
                        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, block_size);
   return LAUNCH_OK();

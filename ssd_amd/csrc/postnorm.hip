@@ -51,7 +51,8 @@ embed_hist_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, 
 }
 
 // One token row per workgroup.  v = the sublayer's fp32 output row, or the routed mix sum_j wt[t][j] * ydn[inv[t * top + j]] in slot
-// order (computed twice, the same arithmetic both times: once for the statistic, once for the sum);  x += w * v / sqrt(mean(v^2) + eps).
+// order (kept in registers between the statistic and the sum for rows of up to 16 entries per thread, else computed twice with the
+// same arithmetic);  x += w * v / sqrt(mean(v^2) + eps).
 // With a history: level n - 1 receives x and x becomes sum_(j < n) coef[j] * level_j (j ascending; the newest level from registers).
 template <typename T, int NT>
 __global__ void __launch_bounds__(NT)
@@ -67,12 +68,24 @@ postnorm_tail_kernel(const float* __restrict__ y, const float* __restrict__ ydn,
     for (int j = 0; j < top; ++j) v = fmaf(wt[t * top + j], ydn[(size_t)inv[t * top + j] * W + c], v);
     return v;
   };
+  constexpr int KEEP = 16;
+  const bool kept = W <= KEEP * NT;
+  float vk[KEEP];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += NT) { const float v = val(c); ss += v * v; }
+  if (kept) {
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      const int c = threadIdx.x + k * NT;
+      vk[k] = c < W ? val(c) : 0.f;
+      ss += vk[k] * vk[k];
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) { const float v = val(c); ss += v * v; }
+  }
   ss = block_sum<NT>(ss, red);
   const float r = 1.0f / sqrtf(ss / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += NT) {
-    float v = xr[c] + val(c) * r * w[c];
+  auto finish = [&](int c, float yv) {
+    float v = xr[c] + yv * r * w[c];
     if (hist) {
       hist[(size_t)(n - 1) * hist_stride + t * W + c] = v;
       float a = 0.f;
@@ -81,6 +94,15 @@ postnorm_tail_kernel(const float* __restrict__ y, const float* __restrict__ ydn,
     }
     xr[c] = v;
     if (next_out) stf<T>(next_out + t * W + c, v);
+  };
+  if (kept) {
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      const int c = threadIdx.x + k * NT;
+      if (c < W) finish(c, vk[k]);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) finish(c, val(c));
   }
 }
 
