@@ -67,14 +67,6 @@ winattn_store_kernel(const float* __restrict__ qkv, long ld, float eps, const in
   }
 }
 
-__device__ __forceinline__ float block_sum_256(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
-}
-
 // q' = w_q * q / rms(q) over all H * D entries (k alike over G * D), then per head the pair (i, i + half) turns by pos * qk_freqs[i];
 // v heads turn over all Dv entries by pos * v_freqs[i] (v_freqs NULL: stored as they are).  grid = (tokens, column blocks): every
 // workgroup of a token sums the squares of the whole row itself (a few thousand cached floats) and takes a share of the work items --
@@ -85,7 +77,7 @@ winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __res
                           const int64_t* __restrict__ positions, const float* __restrict__ qk_freqs, int rot_dims,
                           const float* __restrict__ v_freqs, const int32_t* __restrict__ slots, T* __restrict__ q_out,
                           T* __restrict__ kc, T* __restrict__ vc, int H, int G, int D, int Dv, int bs) {
-  __shared__ float red[4];
+  __shared__ float red[8];
   const int t = blockIdx.x;
   const int Nq = H * D, Nk = G * D;
   const float* row = qkv + (size_t)t * ld;
@@ -96,8 +88,12 @@ winattn_store_rope_kernel(const float* __restrict__ qkv, long ld, const T* __res
   float sq = 0.f, sk = 0.f;
   for (int i = threadIdx.x; i < Nq; i += 256) { const float v = row[i]; sq += v * v; }
   for (int i = threadIdx.x; i < Nk; i += 256) { const float v = row[Nq + i]; sk += v * v; }
-  sq = block_sum_256(sq, red);
-  sk = block_sum_256(sk, red);
+  sq = wave_sum(sq);                                       // both statistics through one pair of barriers
+  sk = wave_sum(sk);
+  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = sq; red[4 + (threadIdx.x >> 6)] = sk; }
+  __syncthreads();
+  sq = (red[0] + red[1]) + (red[2] + red[3]);
+  sk = (red[4] + red[5]) + (red[6] + red[7]);
   const float rq = 1.0f / sqrtf(sq / (float)Nq + eps), rk = 1.0f / sqrtf(sk / (float)Nk + eps);
   const int half = rot_dims >> 1, per = D - half;          // items of a q / k head: `half` pairs, then the entries that do not turn
   const int hv = Dv >> 1, perv = v_freqs ? hv : Dv;        // items of a v head
@@ -238,8 +234,8 @@ winattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T*
       float o = 0.f;
       for (int w = 0; w < 4; ++w) o += sacc[w * Dv + dp] * f[w];
       o = o / L;
-      const float ang = (float)pos * out_freqs[d < hv ? d : d - hv];
-      const float c = cosf(ang), sn = sinf(ang);
+      float sn, c;
+      sincosf((float)pos * out_freqs[d < hv ? d : d - hv], &sn, &c);
       s = d < hv ? s * c + o * sn : s * c - o * sn;
     }
     stf<T>(out + ((size_t)t * H + h) * Dv + d, s);
@@ -435,8 +431,8 @@ winattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
       for (int i = 0; i < MV / 2; ++i)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float ang = (float)pos * out_freqs[i * 16 + qd * 4 + e];
-          const float c = cosf(ang), sn = sinf(ang);
+          float sn, c;
+          sincosf((float)pos * out_freqs[i * 16 + qd * 4 + e], &sn, &c);
           const float a = acc[i][e], b = acc[i + MV / 2][e];
           acc[i][e] = a * c + b * sn;
           acc[i + MV / 2][e] = b * c - a * sn;
@@ -451,8 +447,8 @@ winattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc,
           f32x4_t na, nb;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float ang = (float)pos * out_freqs[i * 16 + qd * 4 + e];
-            const float c = cosf(ang), sn = sinf(ang);
+            float sn, c;
+            sincosf((float)pos * out_freqs[i * 16 + qd * 4 + e], &sn, &c);
             na[e] = acc[i][e] * c + pb[e] * sn;
             nb[e] = pb[e] * c - acc[i][e] * sn;
           }

@@ -135,8 +135,8 @@ rope_rows_kernel(float* __restrict__ rows, long ld, const int64_t* __restrict__ 
     float* p = rows + t * ld + (blk ? off_b : off_a) + h * D;
     const float sc = blk ? scale_b : scale_a;
     if (i < half) {
-      const float ang = pos * freqs[i];
-      const float c = cosf(ang), s = sinf(ang);
+      float s, c;
+      sincosf(pos * freqs[i], &s, &c);
       const float a = p[i], b = p[i + half];
       p[i] = (a * c - b * s) * sc;
       p[i + half] = (b * c + a * s) * sc;
