@@ -94,7 +94,7 @@ def configs():
         "fast_forms": F.make_config([A(heads=8, kv_heads=2, dim=32, vdim=64, window=70, mlp=D(48)),
                                      R(heads=2, dim=32, vdim=32, mlp=M(experts=4, top=2, ff=16)),
                                      L(heads=4, dim=16, rot_dim=32, vdim=16, kv_rank=64, mlp=D(48)),
-                                     A(heads=4, kv_heads=4, dim=64, vdim=32, window=40, rot_dims=32),
+                                     A(heads=4, kv_heads=4, dim=64, vdim=32, window=44, rot_dims=32),
                                      R(heads=1, dim=64, vdim=64, rot_dims=16), L(heads=20, dim=8, rot_dim=32, vdim=8, kv_rank=96, rot_dims=16),
                                      A(heads=20, kv_heads=1, dim=32, vdim=96, window=0, mlp=M(experts=4, top=1, ff=16, groups=2, keep=2))],
                                     vocab=120, width=96),

@@ -108,7 +108,7 @@ def test_gate_rows(f32):
     assert torch.allclose(out.cpu().double(), o[:, :N].double() * torch.sigmoid(g[:, :N].double()), **tol(f32))
 
 
-@pytest.mark.parametrize("E,top,groups,keep", [(12, 4, 2, 1), (12, 3, 4, 2), (6, 2, 1, 1), (8, 8, 2, 2), (9, 2, 9, 3), (5, 1, 5, 1), (64, 6, 8, 3)])
+@pytest.mark.parametrize("E,top,groups,keep", [(10, 4, 2, 1), (12, 3, 4, 2), (6, 2, 1, 1), (8, 8, 2, 2), (9, 2, 9, 3), (5, 1, 5, 1), (64, 6, 8, 3)])
 def test_grouped_sigmoid_router_with_choice_correction(E, top, groups, keep):
     """Corrections large enough that the choice differs from the plain scores' order, and negative enough that choice scores of whole
     groups are negative (an excluded expert must count as -inf, not 0)."""
@@ -205,7 +205,7 @@ def attention_reference(q, k, v, wq, wk, sinks, window, scale, eps, dims, base):
 ATT_CASES = [
     # f32, H, G, D, Dv, window, rot dims, block, MFMA form
     (True, 4, 2, 12, 6, 7, 8, 16, False), (True, 3, 1, 24, 10, 33, 24, 16, False), (True, 2, 2, 8, 4, 0, 0, 16, False),
-    (False, 4, 2, 12, 6, 7, 8, 16, False), (False, 8, 2, 32, 64, 40, 32, 32, True), (False, 4, 4, 64, 32, 70, 16, 64, True),
+    (False, 4, 2, 12, 6, 7, 8, 16, False), (False, 8, 2, 32, 64, 44, 32, 32, True), (False, 4, 4, 64, 32, 70, 16, 64, True),
     (False, 6, 1, 32, 96, 0, 32, 32, True), (False, 2, 1, 128, 128, 50, 64, 32, True), (False, 2, 2, 32, 32, 1, 32, 32, True),
 ]
 
