@@ -190,7 +190,7 @@ FAMILY_SOURCES = {
     "fatulix": _COMMON_ROWS + ["attention_diff.hip"],
     "zerusun": _COMMON_ROWS + ["dyt.hip", "attention_latent.hip", "lightning.hip"],
     "fomunex": _COMMON_ROWS + ["prenorm.hip", "attention_window.hip", "recurrent.hip"],
-    "dosuvik": _COMMON_ROWS + ["postnorm.hip", "prenorm.hip", "attention_window.hip", "attention_latent.hip", "lightning.hip",
+    "dosuvik": _COMMON_ROWS + ["postnorm.hip", "prenorm.hip", "dyt.hip", "attention_window.hip", "attention_latent.hip", "lightning.hip",
                                "recurrent.hip"],
 }
 

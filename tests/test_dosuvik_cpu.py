@@ -237,3 +237,30 @@ def test_bench_option_and_equal_size_pairs():
         rd, rz = dos.layers[1].mixer, zer.layers[1].mixer
         assert (rd.heads, rd.dim, rd.vdim) == (rz.heads, rz.dim, rz.vdim)
         assert dict(param_shapes(dos))["l3.dwa"] == (5,)
+
+
+def test_family_libraries_hold_every_entry_point_their_model_calls():
+    """A checkout without a built library compiles only the translation units of the model's family (hip/lib.py FAMILY_SOURCES): every
+    wrapper a family's model file (and the base class they share) calls must bind a symbol that one of those units defines -- in
+    both element modes, also on branches a quick run does not take."""
+    import os
+    import re
+    from ssd_amd.hip.lib import FAMILY_SOURCES
+    from tests.conftest import ROOT
+    ops = open(os.path.join(ROOT, "ssd_amd", "hip", "ops.py")).read()
+    symbol_of = {}
+    for m in re.finditer(r"^def (\w+)\(.*?(?=^def |\Z)", ops, flags=re.M | re.S):
+        syms = re.findall(r"\.(ssd_\w+)\(", m.group(0))
+        if syms:
+            symbol_of[m.group(1)] = syms
+    base = open(os.path.join(ROOT, "ssd_amd", "res32.py")).read()
+    for family, sources in FAMILY_SOURCES.items():
+        defined = set()
+        for f in sources:
+            defined |= set(re.findall(r'extern "C" int (ssd_\w+)\(', open(os.path.join(ROOT, "ssd_amd", "csrc", f)).read()))
+        model = open(os.path.join(ROOT, "ssd_amd", family + ".py")).read()
+        used = set(re.findall(r"\bH\.(\w+)\(", model + base))
+        assert used, family
+        for op in sorted(used):
+            for sym in symbol_of[op]:
+                assert sym in defined, f"{family}: H.{op} needs {sym}, which none of {sources} defines"
