@@ -309,6 +309,31 @@ def test_bf16_fast_forms_through_the_engine_portions_decoding_and_mixed_steps(tm
     assert close(torch.cat(ga), ra, "bfloat16", fa) and close(torch.cat(gb), rb, "bfloat16", fb)
 
 
+def test_bf16_fast_forms_over_a_long_context_without_windows(tmp_path):
+    """Hundreds of keys per row through the MFMA attentions with no window at all (the latent attention's key slices over the grid, the
+    grouped-query attention's wave split), a prompt of many pages, then decoding: against the oracle and against the scalar forms."""
+    R, L, A, D, M = F.retention_layer, F.latent_layer, F.attention_layer, F.dense_mlp, F.moe_mlp
+    cfg = F.make_config([L(heads=4, dim=16, rot_dim=32, vdim=16, kv_rank=64, mlp=D(48)),
+                         A(heads=4, kv_heads=2, dim=32, vdim=32, window=0, rot_dims=16, mlp=M(experts=4, top=2, ff=16, groups=2, keep=1)),
+                         R(heads=2, dim=32, vdim=32, decay=[0.99, 0.999], mlp=None)], vocab=90, width=64)
+    w = F.random_model(cfg, 21)
+    n = 700
+    toks = tokens(n, cfg["vocab"], 22)
+    ref = F.forward(cfg, w, toks)
+    fl = floor16(cfg, w, toks, ref)
+    cuts = [600] + list(range(601, 641)) + [n]
+    eng = engine(tmp_path, cfg, w, "bfloat16", max_tokens=768, block_size=64)
+    assert all(eng.runner.model.mfma.values())
+    got = _replay(eng, "a", toks, cuts)
+    assert close(got, ref, "bfloat16", fl), rel_err(got, ref)
+    eng.runner.model.scalar_attention = True
+    scalar = _replay(eng, "s", toks, cuts)
+    assert row_err(got, scalar.double().cpu()).median() < 0.02
+    eng32 = engine(tmp_path / "f", cfg, w, "float32", max_tokens=768, block_size=64)
+    got32 = _replay(eng32, "a", toks, cuts)
+    assert close(got32, ref, "float32", oracle(cfg, w, toks)[1]), rel_err(got32, ref)
+
+
 def test_fast_forms_in_fp32_rows_equal_for_any_cut(tmp_path):
     """The register scan also runs in the fp32 element mode; its rows do not depend on the cut either."""
     cfg, w = make("fast_forms", seed=10)

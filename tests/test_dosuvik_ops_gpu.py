@@ -36,9 +36,10 @@ d = lambda t: t.to(DEV).contiguous()
 
 
 @pytest.mark.parametrize("f32", [True, False])
-@pytest.mark.parametrize("W,T", [(40, 9), (328, 9), (2304, 5)])
+# the last case: a row too wide for the registers that keep the routed mix between the statistic and the sum (it is computed twice)
+@pytest.mark.parametrize("W,T", [(40, 9), (328, 9), (2304, 5), (4352, 70)])
 def test_embedding_rows_output_norm_tail_and_depth_average(f32, W, T):
-    V, top, eps, levels, Tmax = 23, 3, 1e-5, 4, 16
+    V, top, eps, levels, Tmax = 23, 3, 1e-5, 4, T + 7
     el = elem(f32)
     table = rnd(V, W, seed=1).to(el)
     ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(4))
